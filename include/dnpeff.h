@@ -1,0 +1,315 @@
+/*
+ * dnpeff.h -- C ABI of the MI355X D-NPEFF NMF library (libdnpeff_hip.so).
+ *
+ * Plain pointers and sizes only.  Every function returns 0 on success and a
+ * non-zero status on failure; dnpeff_last_error() then holds a message.  The
+ * reference aborts the process on every error (print + bare `throw;`,
+ * cc/cuda_d_npeff/src/cuda/cuda_statuses.h:15-38); hosts that want that
+ * behaviour turn a non-zero status into message + abort.
+ *
+ * Storage conventions
+ *   - A is CSR with 64-bit row offsets and 32-bit column ids.
+ *   - Host-visible W is [n, r] row-major, host-visible H is [r, m] row-major:
+ *     the layouts the reference writes to "data/W" and "data/H"
+ *     (cc/cuda_d_npeff/src/io/nmf_decomp_h5.h:38-56).
+ *   - On the device both factors are kept "tall and skinny" with the r
+ *     components of one row/column contiguous: W as [n, r], H as [m, r].
+ *     [m, r] row-major is byte-for-byte the reference's column-major r x m H
+ *     (multi_mu_dense_factors_device_contexts1.h:158).  Entry points that take
+ *     device factor pointers (dnpeff_op_*) use this device layout.
+ *
+ * Threading: handles are not thread safe; one host thread drives one handle.
+ * All work of the library runs on one HIP stream of default priority.
+ */
+#ifndef DNPEFF_H_
+#define DNPEFF_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dnpeff_csr dnpeff_csr; /* device-resident CSR matrix + loader state   */
+typedef struct dnpeff_nmf dnpeff_nmf; /* dense-factor MU NMF (MuNmf + DeviceContext)  */
+typedef struct dnpeff_fit dnpeff_fit; /* fixed sparse-H, W-only learner (Learner)     */
+
+/* ------------------------------------------------------------------------- */
+/* Library state                                                              */
+/* ------------------------------------------------------------------------- */
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* dnpeff_last_error(void);
+
+/* Number of visible GPUs.  Replaces cudaGetDeviceCount at
+ * cc/cuda_d_npeff/mains/run_nmf_on_pefs.cu:126 and Cuda::GetDeviceCount at
+ * cc/cuda_d_npeff/mains/fit_coeffs_to_sparse_H.cu:74-78. */
+int dnpeff_device_count(int* count);
+
+/* Name and total memory of device 0. */
+int dnpeff_device_info(char* name, int name_len, int64_t* total_bytes, int* n_cus);
+
+/* Block until everything queued on the library's stream has finished
+ * (cudaStreamSynchronize, multi_mu_dense_factors_nmf1.h:351-356). */
+int dnpeff_sync(void);
+
+/* Library stream as a hipStream_t, for callers that order their own work. */
+void* dnpeff_stream(void);
+
+/* Plain device buffers for callers of the dnpeff_op_* entry points that have
+ * no device allocator of their own (DeviceCudaContext::dmalloc / dfree and the
+ * copies of cc/cuda_d_npeff/src/cuda/cuda_context.h:58-69, transfers.h).
+ * Copies wait for the library stream first and are synchronous. */
+int dnpeff_dev_malloc(int64_t bytes, void** out);
+int dnpeff_dev_free(void* p);
+int dnpeff_dev_upload(void* dst_dev, const void* src_host, int64_t bytes);
+int dnpeff_dev_download(void* dst_host, const void* src_dev, int64_t bytes);
+
+/* ------------------------------------------------------------------------- */
+/* Loader: CSR on the device, row normalisation, column compaction            */
+/* ------------------------------------------------------------------------- */
+
+/* Upload a host CSR matrix.  Replaces ElCsrMatrix<IndT> + moveAToDeviceAsync
+ * (cc/cuda_d_npeff/src/util/matrices.h:172-199;
+ * multi_mu_dense_factors_device_contexts1.h:182-195).  Column ids inside a row
+ * need not be sorted.  Host buffers are only read during the call. */
+int dnpeff_csr_from_host(int64_t n_rows, int64_t n_cols, int64_t nnz,
+                         const int64_t* rowptr, const int32_t* colind,
+                         const float* vals, dnpeff_csr** out);
+
+/* Build the CSR matrix of a fixed-width PEF block: values/indices are
+ * [n_rows, k] row-major, row offsets are i*k.  Replaces
+ * PefSparseFishers<IndT>::read's construction
+ * (cc/cuda_d_npeff/src/io/pef_fisher_h5.h:170-177). */
+int dnpeff_csr_from_pef(int64_t n_rows, int64_t k, int64_t dense_fisher_size,
+                        const int32_t* indices, const float* values,
+                        dnpeff_csr** out);
+
+/* vals[row] /= (norms[row] + eps), fp32.  Replaces normalizeFishers_inPlace
+ * (cc/cuda_d_npeff/src/io/pef_fisher_h5.h:38-52; eps default 1e-9f there). */
+int dnpeff_csr_normalize_rows(dnpeff_csr* A, const float* norms_host, float eps);
+
+/* Drop every column with fewer than min_count entries and renumber the rest in
+ * ascending original order; entries of dropped columns are removed, in-row
+ * order is kept.  Bit-exact replacement of removeSmallestL0NormColumns_inPlace
+ * (cc/cuda_d_npeff/src/util/sparse_util.h:78-159).  Afterwards
+ * dnpeff_csr_kept_indices returns newToOgIndex. */
+int dnpeff_csr_compact_columns(dnpeff_csr* A, int min_count);
+
+/* Keep only entries whose column id appears in kept[0..n_kept) and renumber
+ * them to their position in kept.  Bit-exact replacement of
+ * Cuda::Host::CsrMatrix::RetainColumns_InPlace
+ * (cc/cuda_d_npeff/src/cuda/host/sparse_matrix.h:141-170). */
+int dnpeff_csr_retain_columns(dnpeff_csr* A, const int32_t* kept, int64_t n_kept);
+
+int dnpeff_csr_shape(const dnpeff_csr* A, int64_t* n_rows, int64_t* n_cols, int64_t* nnz);
+
+/* Column count before the last compaction (fisherDenseSize,
+ * cc/cuda_d_npeff/mains/run_nmf_on_pefs.cu:174). */
+int dnpeff_csr_full_dense_size(const dnpeff_csr* A, int64_t* out);
+
+/* Copy the matrix back: rowptr[n_rows+1], colind[nnz], vals[nnz]; any pointer
+ * may be NULL to skip that array. */
+int dnpeff_csr_download(const dnpeff_csr* A, int64_t* rowptr, int32_t* colind, float* vals);
+
+/* newToOgIndex[n_cols] of the last compact/retain call (identity if none). */
+int dnpeff_csr_kept_indices(const dnpeff_csr* A, int32_t* new_to_og);
+
+/* Sum of squares of all values, accumulated in fp64.  Replaces
+ * computeASqNorm (multi_mu_dense_factors_device_contexts1.h:274-294) and
+ * ComputeAndAccumulate_SquaredNormA (nmf/sparse2/nmf_sparse_H.h:250-262). */
+int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out);
+
+/* Build (once) the transposed CSR on the device: column offsets, and per
+ * column the (row, value) pairs in ascending row order.  Deterministic
+ * replacement of CsrTranspose (cc/cuda_d_npeff/src/cuda/ops/transpose.h:170-439). */
+int dnpeff_csr_build_transpose(dnpeff_csr* A);
+
+/* Copy the transposed CSR back: colptr[n_cols+1], rowind[nnz], vals[nnz]. */
+int dnpeff_csr_download_transpose(dnpeff_csr* A, int64_t* colptr, int32_t* rowind, float* vals);
+
+/* Release the arrays that only dnpeff_op_spmm_n / dnpeff_nmf_* need (row-major
+ * copy) or only spmm_t needs (transposed copy).  which: 1 = row-major copy,
+ * 2 = transposed copy. */
+int dnpeff_csr_release(dnpeff_csr* A, int which);
+
+int dnpeff_csr_destroy(dnpeff_csr* A);
+
+/* Contiguous split sizes: total/n_splits each, remainder added to the last.
+ * Replaces getSizeOfSplit (cc/cuda_d_npeff/src/util/matrix_util.h:10-21) and
+ * CsrMatrix::GetSizeOfSplit (cuda/host/sparse_matrix.h:107-117).  Returns -1
+ * for split_index >= n_splits (the reference throws). */
+int64_t dnpeff_size_of_split(int64_t total, int64_t n_splits, int64_t split_index);
+
+/* ------------------------------------------------------------------------- */
+/* Synthetic PEF generator (benchmark / test inputs, not part of the reference)*/
+/* ------------------------------------------------------------------------- */
+
+/* Per row i: k_i distinct column ids by successive Zipf(s) draws over
+ * [0, n_cols) rejecting duplicates, draw order kept; values exp(N(mu, sigma^2))
+ * in fp32.  k_i = k_fixed, or, when k_min > 0, round(exp(U(ln k_min, ln k_max))).
+ * norms_out_host[n_rows] (may be NULL) receives the fp32 L2 norm of each row
+ * so that dnpeff_csr_normalize_rows L2-normalises it. */
+int dnpeff_synth_pef(int64_t n_rows, int64_t n_cols, int64_t k_fixed,
+                     int64_t k_min, int64_t k_max, double zipf_s,
+                     double mu, double sigma, uint64_t seed,
+                     float* norms_out_host, dnpeff_csr** out);
+
+/* Same generator on the host, one thread; arrays sized by the caller
+ * (rowptr[n_rows+1] is written first when colind == NULL so the caller can
+ * size colind/vals). */
+int dnpeff_synth_pef_host(int64_t n_rows, int64_t n_cols, int64_t k_fixed,
+                          int64_t k_min, int64_t k_max, double zipf_s,
+                          double mu, double sigma, uint64_t seed,
+                          int64_t* rowptr, int32_t* colind, float* vals,
+                          float* norms);
+
+/* U[0,1) initial factor value of logical element (row, col) of matrix
+ * matrix_id (0 = W [n, r], 1 = H [r, m]); host mirror of the device
+ * initialiser.  Replaces curandGenerateUniform
+ * (multi_mu_dense_factors_device_contexts1.h:197-207). */
+float dnpeff_uniform_at(uint64_t seed, int matrix_id, int64_t row, int64_t col, int64_t n_cols);
+
+/* ------------------------------------------------------------------------- */
+/* Dense-factor MU NMF (run_nmf_on_pefs hot loop)                             */
+/* ------------------------------------------------------------------------- */
+
+/* Create the context for A ~= W H with W [n, r], H [r, m].  Builds the
+ * transposed CSR, allocates W, H and one [max(n, m), r] scratch, computes
+ * ||A||^2.  A stays owned by the caller and must outlive the context.
+ * Replaces MuNmf<IndT>::MuNmf + DeviceContext ctor
+ * (multi_mu_dense_factors_nmf1.h:81-122;
+ * multi_mu_dense_factors_device_contexts1.h:129-170,384-434).
+ * Like the reference it refuses n_rows > n_cols. */
+int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out);
+
+/* W then H ~ U[0,1) from the seed (initializeW / initializeH,
+ * multi_mu_dense_factors_device_contexts1.h:197-233). */
+int dnpeff_nmf_init_factors(dnpeff_nmf* nmf);
+
+/* Load caller-chosen factors: W [n, r] row-major, H [r, m] row-major (either
+ * may be NULL to keep the current one). */
+int dnpeff_nmf_set_factors(dnpeff_nmf* nmf, const float* W_nr, const float* H_rm);
+
+/* n_steps iterations of: W-update, then H-update with the new W
+ * (MuNmf::run loop body, multi_mu_dense_factors_nmf1.h:175-182).  Returns
+ * without waiting for the device. */
+int dnpeff_nmf_step(dnpeff_nmf* nmf, int n_steps);
+
+/* W <- W * (A H^T) / (W (H H^T) + eps)   (updateW, nmf1.h:293-305). */
+int dnpeff_nmf_update_W(dnpeff_nmf* nmf);
+/* H <- H * (W^T A) / ((W^T W) H + eps)   (updateH, device_contexts1.h:296-309). */
+int dnpeff_nmf_update_H(dnpeff_nmf* nmf);
+
+/* sqrt(||A||^2 + <W^T W, H H^T> - 2 <A H^T, W>) with fp64 accumulation of the
+ * reductions: the quantity of computeUncachedLoss (nmf1.h:242-274,
+ * device_contexts1.h:337-354) through the same trace identity. */
+int dnpeff_nmf_loss(dnpeff_nmf* nmf, double* out);
+
+/* The three terms of the loss: ||A||^2, <H,(W^T W)H>, <W^T A,H>. */
+int dnpeff_nmf_loss_terms(dnpeff_nmf* nmf, double* sq_norm_A, double* pos, double* neg);
+
+/* Copy the factors to the host in the output-file layout: W [n, r] row-major
+ * (loadWToHostSync + toRowMajor_inPlace, nmf1.h:207-220, matrices.h:49-62),
+ * H [r, m] row-major (loadHToHostSync + toRowMajor_inPlace, nmf1.h:222-240). */
+int dnpeff_nmf_get_W(dnpeff_nmf* nmf, float* W_nr);
+int dnpeff_nmf_get_H(dnpeff_nmf* nmf, float* H_rm);
+
+/* Device pointers of W [n, r] and H [m, r] (device layout). */
+int dnpeff_nmf_device_factors(dnpeff_nmf* nmf, void** W_dev, void** H_dev);
+
+/* Per-kernel timing with HIP events on the library stream.  enable != 0 turns
+ * it on for subsequent steps; dnpeff_nmf_timings waits for the stream and
+ * returns, per kernel class, summed milliseconds and launch counts since the
+ * last reset.  Classes (DNPEFF_K_*) below. */
+enum {
+  DNPEFF_K_SPMM_N = 0,   /* A H^T                     */
+  DNPEFF_K_SPMM_N_REDUCE = 1,
+  DNPEFF_K_GRAM_H = 2,   /* H H^T  (k = m)            */
+  DNPEFF_K_XG_MU_W = 3,  /* W (H H^T) fused with MU   */
+  DNPEFF_K_SPMM_T = 4,   /* A^T W                     */
+  DNPEFF_K_GRAM_W = 5,   /* W^T W  (k = n)            */
+  DNPEFF_K_XG_MU_H = 6,  /* (W^T W) H fused with MU   */
+  DNPEFF_K_COUNT = 7
+};
+int dnpeff_nmf_set_profiling(dnpeff_nmf* nmf, int enable);
+int dnpeff_nmf_timings(dnpeff_nmf* nmf, double* ms_sum /*[DNPEFF_K_COUNT]*/,
+                       int64_t* launches /*[DNPEFF_K_COUNT]*/, int reset);
+
+int dnpeff_nmf_destroy(dnpeff_nmf* nmf);
+
+/* ------------------------------------------------------------------------- */
+/* Fixed sparse H, W-only learner (fit_coeffs_to_sparse_H)                    */
+/* ------------------------------------------------------------------------- */
+
+/* Stage 1: H H^T (r x r) and A H^T (n x r) from sparse A [n, m] and sparse H
+ * [r, m], plus ||A||^2.  Replaces Learner::RunFirstStage
+ * (cc/cuda_d_npeff/src/nmf/sparse2/nmf_sparse_H.h:157-292;
+ * cuda/ops/spsp_matmul.h:95-131).  A and H may be destroyed afterwards. */
+int dnpeff_fit_create(dnpeff_csr* A, dnpeff_csr* H, float eps, int64_t seed, dnpeff_fit** out);
+
+/* W ~ U[0,1) from the seed / caller-chosen W [n, r] row-major. */
+int dnpeff_fit_init_W(dnpeff_fit* fit);
+int dnpeff_fit_set_W(dnpeff_fit* fit, const float* W_nr);
+
+/* n_steps of WHH = W (H H^T); W <- W * (A H^T) / (WHH + eps)
+ * (DoMuStep, nmf_sparse_H.h:342-345). */
+int dnpeff_fit_step(dnpeff_fit* fit, int n_steps);
+
+/* reference_loss: sqrt(||A||^2 + <WHH, W> - 2 <A H^T, W>) with WHH as left by
+ * the last step, i.e. computed from W before that step's update -- the value
+ * the reference logs (nmf_sparse_H.h:319-331).  true_loss uses W (H H^T) of
+ * the current W.  Either pointer may be NULL. */
+int dnpeff_fit_loss(dnpeff_fit* fit, double* reference_loss, double* true_loss);
+
+int dnpeff_fit_get_W(dnpeff_fit* fit, float* W_nr);
+/* Stage-1 products: AH [n, r] row-major, HH [r, r]. */
+int dnpeff_fit_get_products(dnpeff_fit* fit, float* AH_nr, float* HH_rr, double* sq_norm_A);
+int dnpeff_fit_destroy(dnpeff_fit* fit);
+
+/* ------------------------------------------------------------------------- */
+/* Single kernels on device pointers (parity tests and profiling)             */
+/* All factor pointers are device memory in the device layout ([rows, r]).    */
+/* They are queued on the library stream; call dnpeff_sync() before reading.  */
+/* ------------------------------------------------------------------------- */
+
+/* F[i] *= num[i] / (den[i] + eps), i < count.  kernelNmfMuUpdate
+ * (cc/cuda_d_npeff/src/nmf/sparse/kernels.h:24-34) and
+ * MultiplicativeUpdate_Kernel (nmf/kernels/mu.h:32-38). */
+int dnpeff_op_mu(int64_t count, float* F, const float* num, const float* den, float eps);
+
+/* N[n, r] = A H^T with H given as [m, r].  cusparseSpMM(N, T) at
+ * device_contexts1.h:255-258,317. */
+int dnpeff_op_spmm_n(dnpeff_csr* A, int r, const float* H_mr, float* N_nr);
+
+/* T[m, r] = A^T W with W [n, r]; needs dnpeff_csr_build_transpose.
+ * cusparseSpMM(T, T) at device_contexts1.h:260-265,301. */
+int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
+
+/* G[r, r] = X^T X for X [rows, r].  cublasSgemm at device_contexts1.h:303,322. */
+int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr);
+
+/* out = X * num / (X G + eps) with X, num, out [rows, r], G [r, r] symmetric.
+ * out may alias num but not X.  D_out (may be NULL) receives X G.
+ * cublasSgemm + kernelNmfMuUpdate at device_contexts1.h:306-308,329-332. */
+int dnpeff_op_xg_mu(int64_t rows, int r, const float* X, const float* G_rr,
+                    const float* num, float eps, float* out, float* D_out);
+
+/* <x, y> over count floats, fp64 accumulation; result to the host.
+ * frobeniusProductToHost (device_contexts1.h:503-537). */
+int dnpeff_op_dot(int64_t count, const float* x, const float* y, double* out_host);
+
+/* out[n, r] = A B^T for sparse A [n, m] and sparse B [r, m] (both CSR); B's
+ * transposed copy is built if missing.  Partitioned_SpSpMatmul_ToDense
+ * (cc/cuda_d_npeff/src/cuda/ops/spsp_matmul.h:95-131). */
+int dnpeff_op_spsp_dense(dnpeff_csr* A, dnpeff_csr* B, float* out_nr);
+
+/* x[i] = U[0,1) value of logical element i of matrix matrix_id, written in the
+ * device layout (see dnpeff_uniform_at). */
+int dnpeff_op_init_uniform(int matrix_id, int64_t logical_rows, int64_t logical_cols,
+                           uint64_t seed, float* x);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DNPEFF_H_ */

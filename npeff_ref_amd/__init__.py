@@ -1,0 +1,38 @@
+"""MI355X-native D-NPEFF NMF hot path.
+
+The product is ``lib/libdnpeff_hip.so`` (hand-written HIP kernels for gfx950
+behind the C ABI of ``include/dnpeff.h``) and the two C++ executables under
+``csrc/host``.  This package is the thin ctypes binding used by the tests and
+by ``bench.py``; it mirrors the reference's driver classes
+(``MuNmf`` -- cc/cuda_d_npeff/src/nmf/sparse/multi_mu_dense_factors_nmf1.h:81-274,
+``Learner`` -- cc/cuda_d_npeff/src/nmf/sparse2/nmf_sparse_H.h:42-345).
+
+There is no CPU fallback: importing :mod:`npeff_ref_amd.binding` raises if the
+library has not been built.
+"""
+
+from .binding import (  # noqa: F401
+    DnpeffError,
+    Csr,
+    DeviceArray,
+    MuNmf,
+    MuNmfParams,
+    Learner,
+    LearnerParams,
+    lib,
+    device_count,
+    size_of_split,
+    uniform_at,
+    synth_pef_host,
+    KERNEL_CLASSES,
+    sync,
+    device_info,
+    op_mu,
+    op_spmm_n,
+    op_spmm_t,
+    op_gram,
+    op_xg_mu,
+    op_dot,
+    op_spsp_dense,
+    op_init_uniform,
+)

@@ -1,0 +1,393 @@
+// Handles of the two hot loops behind the C ABI: the dense-factor MU NMF of
+// run_nmf_on_pefs and the W-only learner of fit_coeffs_to_sparse_H.
+#include "dnpeff_internal.hpp"
+
+#include <cmath>
+#include <utility>
+#include <vector>
+
+using namespace dn;
+
+// ---------------------------------------------------------------------------
+// Per-kernel timing with HIP events on the library stream
+// ---------------------------------------------------------------------------
+struct EventPair {
+  hipEvent_t start = nullptr, stop = nullptr;
+  int cls = 0;
+};
+
+struct Profiler {
+  bool enabled = false;
+  std::vector<EventPair> pool;   // every pair ever created
+  size_t used = 0;               // pairs in flight since the last collect
+  double ms_sum[DNPEFF_K_COUNT] = {0};
+  int64_t launches[DNPEFF_K_COUNT] = {0};
+
+  int begin(int cls) {
+    if (!enabled) return 0;
+    if (used == pool.size()) {
+      EventPair p;
+      DN_HIP(hipEventCreate(&p.start));
+      DN_HIP(hipEventCreate(&p.stop));
+      pool.push_back(p);
+    }
+    pool[used].cls = cls;
+    DN_HIP(hipEventRecord(pool[used].start, stream()));
+    return 0;
+  }
+  int end() {
+    if (!enabled) return 0;
+    DN_HIP(hipEventRecord(pool[used].stop, stream()));
+    used++;
+    if (used >= 4096) return collect();
+    return 0;
+  }
+  int collect() {
+    if (used == 0) return 0;
+    DN_HIP(hipStreamSynchronize(stream()));
+    for (size_t i = 0; i < used; i++) {
+      float ms = 0.0f;
+      DN_HIP(hipEventElapsedTime(&ms, pool[i].start, pool[i].stop));
+      ms_sum[pool[i].cls] += (double)ms;
+      launches[pool[i].cls] += 1;
+    }
+    used = 0;
+    return 0;
+  }
+  void reset() {
+    for (int i = 0; i < DNPEFF_K_COUNT; i++) {
+      ms_sum[i] = 0.0;
+      launches[i] = 0;
+    }
+  }
+  ~Profiler() {
+    for (auto& p : pool) {
+      if (p.start) (void)hipEventDestroy(p.start);
+      if (p.stop) (void)hipEventDestroy(p.stop);
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Dense-factor MU NMF
+// ---------------------------------------------------------------------------
+struct dnpeff_nmf {
+  dnpeff_csr* A = nullptr;
+  int r = 0;
+  float eps = 0.0f;
+  uint64_t seed = 0;
+  int64_t n = 0, m = 0;
+  float* W = nullptr;        // [n, r]
+  float* W2 = nullptr;       // [n, r] output buffer of the W update
+  float* Nw = nullptr;       // [n, r] A H^T
+  float* H = nullptr;        // [m, r]
+  float* S = nullptr;        // [m, r] A^T W, then the updated H
+  float* G = nullptr;        // [r, r]
+  float* G2 = nullptr;       // [r, r]
+  float* gram_ws = nullptr;  // slice partials of the Gram kernel
+  double* dot_ws = nullptr;  // DOT_BLOCKS partials + 2 results
+  double sq_norm_A = 0.0;
+  Profiler prof;
+};
+
+DN_API int dnpeff_nmf_destroy(dnpeff_nmf* nmf) {
+  if (!nmf) return 0;
+  (void)hipStreamSynchronize(stream());
+  dfree(nmf->W); dfree(nmf->W2); dfree(nmf->Nw); dfree(nmf->H); dfree(nmf->S);
+  dfree(nmf->G); dfree(nmf->G2); dfree(nmf->gram_ws); dfree(nmf->dot_ws);
+  delete nmf;
+  return 0;
+}
+
+DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out) {
+  clear_error();
+  DN_CHECK(out != nullptr, "out is NULL");
+  *out = nullptr;
+  DN_CHECK(A != nullptr, "matrix is NULL");
+  DN_CHECK(rank >= 1 && rank <= 1024, "rank %d outside [1, 1024]", rank);
+  // multi_mu_dense_factors_nmf1.h:95-99
+  DN_CHECK(A->n_rows <= A->n_cols, "Error: Not handling matrices with more rows than columns yet.");
+  DN_TRY(dnpeff_csr_build_transpose(A));
+  DN_TRY(csr_ensure_partials(A, rank));
+  dnpeff_nmf* h = new dnpeff_nmf();
+  h->A = A; h->r = rank; h->eps = eps; h->seed = (uint64_t)seed;
+  h->n = A->n_rows; h->m = A->n_cols;
+  const int64_t nr = h->n * rank, mr = h->m * rank;
+  int64_t ws = gram_workspace_floats(h->m, rank);
+  int64_t ws_n = gram_workspace_floats(h->n, rank);
+  if (ws_n > ws) ws = ws_n;
+  int s = dmalloc(&h->W, nr) || dmalloc(&h->W2, nr) || dmalloc(&h->Nw, nr) ||
+          dmalloc(&h->H, mr) || dmalloc(&h->S, mr) || dmalloc(&h->G, (int64_t)rank * rank) ||
+          dmalloc(&h->G2, (int64_t)rank * rank) || dmalloc(&h->gram_ws, ws) ||
+          dmalloc(&h->dot_ws, DOT_BLOCKS + 2);
+  if (!s) s = dnpeff_csr_sq_norm(A, &h->sq_norm_A);
+  if (s) { dnpeff_nmf_destroy(h); return s; }
+  *out = h;
+  return 0;
+}
+
+DN_API int dnpeff_nmf_init_factors(dnpeff_nmf* nmf) {
+  clear_error();
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  DN_TRY(launch_init_uniform(0, nmf->n, nmf->r, nmf->seed, nmf->W));
+  DN_TRY(launch_init_uniform(1, nmf->r, nmf->m, nmf->seed, nmf->H));
+  return 0;
+}
+
+DN_API int dnpeff_nmf_set_factors(dnpeff_nmf* nmf, const float* W_nr, const float* H_rm) {
+  clear_error();
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (W_nr)
+    DN_HIP(hipMemcpy(nmf->W, W_nr, sizeof(float) * nmf->n * nmf->r, hipMemcpyHostToDevice));
+  if (H_rm) {
+    DN_HIP(hipMemcpy(nmf->S, H_rm, sizeof(float) * nmf->m * nmf->r, hipMemcpyHostToDevice));
+    DN_TRY(launch_transpose(nmf->r, nmf->m, nmf->S, nmf->H));
+    DN_HIP(hipStreamSynchronize(stream()));
+  }
+  return 0;
+}
+
+DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
+  DN_CHECK(h != nullptr, "handle is NULL");
+  dnpeff_csr* A = h->A;
+  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N));
+  DN_TRY(launch_spmm_n(A, h->r, h->H, h->Nw, A->partials));
+  DN_TRY(h->prof.end());
+  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N_REDUCE));
+  DN_TRY(launch_spmm_n_reduce(A, h->r, A->partials, h->Nw));
+  DN_TRY(h->prof.end());
+  DN_TRY(h->prof.begin(DNPEFF_K_GRAM_H));
+  DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
+  DN_TRY(h->prof.end());
+  DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_W));
+  DN_TRY(launch_xg_mu(h->n, h->r, h->W, h->G, h->Nw, h->eps, h->W2, nullptr));
+  DN_TRY(h->prof.end());
+  std::swap(h->W, h->W2);
+  return 0;
+}
+
+DN_API int dnpeff_nmf_update_H(dnpeff_nmf* h) {
+  DN_CHECK(h != nullptr, "handle is NULL");
+  dnpeff_csr* A = h->A;
+  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+  DN_TRY(launch_spmm_t(A, h->r, h->W, h->S));
+  DN_TRY(h->prof.end());
+  DN_TRY(h->prof.begin(DNPEFF_K_GRAM_W));
+  DN_TRY(launch_gram(h->n, h->r, h->W, h->G, h->gram_ws));
+  DN_TRY(h->prof.end());
+  DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_H));
+  DN_TRY(launch_xg_mu(h->m, h->r, h->H, h->G, h->S, h->eps, h->S, nullptr));
+  DN_TRY(h->prof.end());
+  std::swap(h->H, h->S);
+  return 0;
+}
+
+DN_API int dnpeff_nmf_step(dnpeff_nmf* nmf, int n_steps) {
+  clear_error();
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  for (int s = 0; s < n_steps; s++) {
+    DN_TRY(dnpeff_nmf_update_W(nmf));
+    DN_TRY(dnpeff_nmf_update_H(nmf));
+  }
+  return 0;
+}
+
+DN_API int dnpeff_nmf_loss_terms(dnpeff_nmf* h, double* sq_norm_A, double* pos, double* neg) {
+  clear_error();
+  DN_CHECK(h != nullptr, "handle is NULL");
+  dnpeff_csr* A = h->A;
+  // neg = <W^T A, H> = <A H^T, W>
+  DN_TRY(launch_spmm_n(A, h->r, h->H, h->Nw, A->partials));
+  DN_TRY(launch_spmm_n_reduce(A, h->r, A->partials, h->Nw));
+  DN_TRY(launch_dot(h->n * h->r, h->Nw, h->W, h->dot_ws, h->dot_ws + DOT_BLOCKS));
+  // pos = <H, (W^T W) H> = <W^T W, H H^T>
+  DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
+  DN_TRY(launch_gram(h->n, h->r, h->W, h->G2, h->gram_ws));
+  DN_TRY(launch_dot((int64_t)h->r * h->r, h->G, h->G2, h->dot_ws, h->dot_ws + DOT_BLOCKS + 1));
+  double res[2];
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(res, h->dot_ws + DOT_BLOCKS, sizeof(double) * 2, hipMemcpyDeviceToHost));
+  if (sq_norm_A) *sq_norm_A = h->sq_norm_A;
+  if (neg) *neg = res[0];
+  if (pos) *pos = res[1];
+  return 0;
+}
+
+DN_API int dnpeff_nmf_loss(dnpeff_nmf* nmf, double* out) {
+  DN_CHECK(out != nullptr, "out is NULL");
+  double a, p, q;
+  DN_TRY(dnpeff_nmf_loss_terms(nmf, &a, &p, &q));
+  *out = std::sqrt(a + p - 2.0 * q);
+  return 0;
+}
+
+DN_API int dnpeff_nmf_get_W(dnpeff_nmf* nmf, float* W_nr) {
+  clear_error();
+  DN_CHECK(nmf && W_nr, "NULL argument");
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(W_nr, nmf->W, sizeof(float) * nmf->n * nmf->r, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+DN_API int dnpeff_nmf_get_H(dnpeff_nmf* nmf, float* H_rm) {
+  clear_error();
+  DN_CHECK(nmf && H_rm, "NULL argument");
+  DN_TRY(launch_transpose(nmf->m, nmf->r, nmf->H, nmf->S));
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(H_rm, nmf->S, sizeof(float) * nmf->m * nmf->r, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+DN_API int dnpeff_nmf_device_factors(dnpeff_nmf* nmf, void** W_dev, void** H_dev) {
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  if (W_dev) *W_dev = nmf->W;
+  if (H_dev) *H_dev = nmf->H;
+  return 0;
+}
+
+DN_API int dnpeff_nmf_set_profiling(dnpeff_nmf* nmf, int enable) {
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  DN_TRY(nmf->prof.collect());
+  nmf->prof.enabled = enable != 0;
+  return 0;
+}
+
+DN_API int dnpeff_nmf_timings(dnpeff_nmf* nmf, double* ms_sum, int64_t* launches, int reset) {
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  DN_TRY(nmf->prof.collect());
+  for (int i = 0; i < DNPEFF_K_COUNT; i++) {
+    if (ms_sum) ms_sum[i] = nmf->prof.ms_sum[i];
+    if (launches) launches[i] = nmf->prof.launches[i];
+  }
+  if (reset) nmf->prof.reset();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Fixed sparse H, W-only learner
+// ---------------------------------------------------------------------------
+struct dnpeff_fit {
+  int64_t n = 0;
+  int r = 0;
+  float eps = 0.0f;
+  uint64_t seed = 0;
+  float* AH = nullptr;   // [n, r]
+  float* HH = nullptr;   // [r, r]
+  float* W = nullptr;    // [n, r]
+  float* W2 = nullptr;   // [n, r]
+  float* WHH = nullptr;  // [n, r] W (H H^T) of the W before the last step
+  float* tmp = nullptr;  // [n, r]
+  double* dot_ws = nullptr;
+  double sq_norm_A = 0.0;
+  bool whh_valid = false;
+};
+
+DN_API int dnpeff_fit_destroy(dnpeff_fit* f) {
+  if (!f) return 0;
+  (void)hipStreamSynchronize(stream());
+  dfree(f->AH); dfree(f->HH); dfree(f->W); dfree(f->W2); dfree(f->WHH); dfree(f->tmp);
+  dfree(f->dot_ws);
+  delete f;
+  return 0;
+}
+
+DN_API int dnpeff_fit_create(dnpeff_csr* A, dnpeff_csr* H, float eps, int64_t seed,
+                             dnpeff_fit** out) {
+  clear_error();
+  DN_CHECK(out != nullptr, "out is NULL");
+  *out = nullptr;
+  DN_CHECK(A && H, "matrix is NULL");
+  DN_CHECK(A->n_cols == H->n_cols, "A has %lld columns but H has %lld", (long long)A->n_cols,
+           (long long)H->n_cols);
+  const int r = (int)H->n_rows;
+  DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
+  dnpeff_fit* f = new dnpeff_fit();
+  f->n = A->n_rows; f->r = r; f->eps = eps; f->seed = (uint64_t)seed;
+  const int64_t nr = f->n * r;
+  int s = dmalloc(&f->AH, nr) || dmalloc(&f->HH, (int64_t)r * r) || dmalloc(&f->W, nr) ||
+          dmalloc(&f->W2, nr) || dmalloc(&f->WHH, nr) || dmalloc(&f->tmp, nr) ||
+          dmalloc(&f->dot_ws, DOT_BLOCKS + 2);
+  if (!s) s = dnpeff_op_spsp_dense(H, H, f->HH);
+  if (!s) s = dnpeff_op_spsp_dense(A, H, f->AH);
+  if (!s) s = dnpeff_csr_sq_norm(A, &f->sq_norm_A);
+  if (!s && hipStreamSynchronize(stream()) != hipSuccess) {
+    set_error("first stage kernels failed");
+    s = 1;
+  }
+  if (s) { dnpeff_fit_destroy(f); return s; }
+  *out = f;
+  return 0;
+}
+
+DN_API int dnpeff_fit_init_W(dnpeff_fit* f) {
+  clear_error();
+  DN_CHECK(f != nullptr, "handle is NULL");
+  f->whh_valid = false;
+  return launch_init_uniform(0, f->n, f->r, f->seed, f->W);
+}
+
+DN_API int dnpeff_fit_set_W(dnpeff_fit* f, const float* W_nr) {
+  clear_error();
+  DN_CHECK(f && W_nr, "NULL argument");
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(f->W, W_nr, sizeof(float) * f->n * f->r, hipMemcpyHostToDevice));
+  f->whh_valid = false;
+  return 0;
+}
+
+DN_API int dnpeff_fit_step(dnpeff_fit* f, int n_steps) {
+  clear_error();
+  DN_CHECK(f != nullptr, "handle is NULL");
+  for (int s = 0; s < n_steps; s++) {
+    DN_TRY(launch_xg_mu(f->n, f->r, f->W, f->HH, f->AH, f->eps, f->W2, f->WHH));
+    std::swap(f->W, f->W2);
+    f->whh_valid = true;
+  }
+  return 0;
+}
+
+DN_API int dnpeff_fit_loss(dnpeff_fit* f, double* reference_loss, double* true_loss) {
+  clear_error();
+  DN_CHECK(f != nullptr, "handle is NULL");
+  const int64_t nr = f->n * f->r;
+  double res[2];
+  // neg = <A H^T, W>
+  DN_TRY(launch_dot(nr, f->AH, f->W, f->dot_ws, f->dot_ws + DOT_BLOCKS));
+  // pos of the current W; W2 receives an update that is discarded
+  DN_TRY(launch_xg_mu(f->n, f->r, f->W, f->HH, f->AH, f->eps, f->W2, f->tmp));
+  DN_TRY(launch_dot(nr, f->tmp, f->W, f->dot_ws, f->dot_ws + DOT_BLOCKS + 1));
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(res, f->dot_ws + DOT_BLOCKS, sizeof(double) * 2, hipMemcpyDeviceToHost));
+  const double neg = res[0], pos_true = res[1];
+  if (true_loss) *true_loss = std::sqrt(f->sq_norm_A + pos_true - 2.0 * neg);
+  if (reference_loss) {
+    double pos_ref = pos_true;
+    if (f->whh_valid) {
+      DN_TRY(launch_dot(nr, f->WHH, f->W, f->dot_ws, f->dot_ws + DOT_BLOCKS));
+      DN_HIP(hipStreamSynchronize(stream()));
+      DN_HIP(hipMemcpy(&pos_ref, f->dot_ws + DOT_BLOCKS, sizeof(double), hipMemcpyDeviceToHost));
+    }
+    *reference_loss = std::sqrt(f->sq_norm_A + pos_ref - 2.0 * neg);
+  }
+  return 0;
+}
+
+DN_API int dnpeff_fit_get_W(dnpeff_fit* f, float* W_nr) {
+  clear_error();
+  DN_CHECK(f && W_nr, "NULL argument");
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(W_nr, f->W, sizeof(float) * f->n * f->r, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+DN_API int dnpeff_fit_get_products(dnpeff_fit* f, float* AH_nr, float* HH_rr, double* sq_norm_A) {
+  clear_error();
+  DN_CHECK(f != nullptr, "handle is NULL");
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (AH_nr) DN_HIP(hipMemcpy(AH_nr, f->AH, sizeof(float) * f->n * f->r, hipMemcpyDeviceToHost));
+  if (HH_rr)
+    DN_HIP(hipMemcpy(HH_rr, f->HH, sizeof(float) * f->r * f->r, hipMemcpyDeviceToHost));
+  if (sq_norm_A) *sq_norm_A = f->sq_norm_A;
+  return 0;
+}

@@ -1,0 +1,785 @@
+// CSR loader on the device: upload, row normalisation, column compaction,
+// column retention, transposed CSR, ||A||^2.  Integer results are bit-exact
+// with the reference's host code; see include/dnpeff.h for the citations.
+#include "dnpeff_internal.hpp"
+
+#include <cstdarg>
+#include <cstring>
+#include <vector>
+
+namespace dn {
+
+// ---------------------------------------------------------------------------
+// Library state
+// ---------------------------------------------------------------------------
+static thread_local char g_error[1024] = "";
+static hipStream_t g_stream = nullptr;
+static int g_n_cus = 0;
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+void clear_error() { g_error[0] = 0; }
+
+hipStream_t stream() {
+  if (!g_stream) {
+    if (hipStreamCreate(&g_stream) != hipSuccess) {
+      fprintf(stderr, "dnpeff: hipStreamCreate failed (no usable GPU?)\n");
+      abort();
+    }
+  }
+  return g_stream;
+}
+
+int n_cus() {
+  if (!g_n_cus) {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, 0) == hipSuccess) g_n_cus = p.multiProcessorCount;
+    if (g_n_cus <= 0) g_n_cus = 256;
+  }
+  return g_n_cus;
+}
+
+// ---------------------------------------------------------------------------
+// Exclusive scan: tile sums -> scan of tile sums -> per-tile scan
+// ---------------------------------------------------------------------------
+constexpr int SCAN_BLOCK = 256;
+constexpr int SCAN_ITEMS = 8;
+constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;
+
+__device__ inline int64_t block_excl_scan(int64_t v, int64_t& total) {
+  __shared__ int64_t sh[SCAN_BLOCK];
+  const int t = threadIdx.x;
+  sh[t] = v;
+  __syncthreads();
+  for (int off = 1; off < SCAN_BLOCK; off <<= 1) {
+    int64_t add = (t >= off) ? sh[t - off] : 0;
+    __syncthreads();
+    sh[t] += add;
+    __syncthreads();
+  }
+  int64_t incl = sh[t];
+  total = sh[SCAN_BLOCK - 1];
+  __syncthreads();
+  return incl - v;
+}
+
+template <class F>
+__global__ void __launch_bounds__(SCAN_BLOCK) k_scan_tile_sums(F f, int64_t n, int64_t* tile_sums) {
+  int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+  int64_t s = 0;
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    int64_t idx = base + i;
+    if (idx < n) s += f(idx);
+  }
+  int64_t total;
+  block_excl_scan(s, total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// In-place exclusive scan of tile_sums[0..n_tiles); tile_sums[n_tiles] = total.
+__global__ void __launch_bounds__(SCAN_BLOCK) k_scan_tiles(int64_t* tile_sums, int64_t n_tiles) {
+  int64_t carry = 0;
+  for (int64_t base = 0; base < n_tiles; base += SCAN_BLOCK) {
+    int64_t idx = base + threadIdx.x;
+    int64_t v = idx < n_tiles ? tile_sums[idx] : 0;
+    int64_t total;
+    int64_t ex = block_excl_scan(v, total);
+    if (idx < n_tiles) tile_sums[idx] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) tile_sums[n_tiles] = carry;
+}
+
+template <class F, class OutT>
+__global__ void __launch_bounds__(SCAN_BLOCK)
+    k_scan_apply(F f, int64_t n, const int64_t* tile_offsets, int64_t n_tiles, OutT* out) {
+  int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+  int64_t v[SCAN_ITEMS];
+  int64_t s = 0;
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    int64_t idx = base + i;
+    v[i] = idx < n ? (int64_t)f(idx) : 0;
+    s += v[i];
+  }
+  int64_t total;
+  int64_t run = block_excl_scan(s, total) + tile_offsets[blockIdx.x];
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    int64_t idx = base + i;
+    if (idx < n) out[idx] = (OutT)run;
+    run += v[i];
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) out[n] = (OutT)tile_offsets[n_tiles];
+}
+
+__global__ void k_set_one_i64(int64_t* p, int64_t v) { *p = v; }
+
+template <class F, class OutT>
+static int exclusive_scan(F f, int64_t n, OutT* out) {
+  hipStream_t st = stream();
+  int64_t n_tiles = ceil_div(n, SCAN_TILE);
+  if (n_tiles == 0) {
+    DN_HIP(hipMemsetAsync(out, 0, sizeof(OutT), st));
+    return 0;
+  }
+  int64_t* tiles = nullptr;
+  DN_TRY(dmalloc(&tiles, n_tiles + 1));
+  hipLaunchKernelGGL((k_scan_tile_sums<F>), dim3((unsigned)n_tiles), dim3(SCAN_BLOCK), 0, st, f, n,
+                     tiles);
+  hipLaunchKernelGGL(k_scan_tiles, dim3(1), dim3(SCAN_BLOCK), 0, st, tiles, n_tiles);
+  hipLaunchKernelGGL((k_scan_apply<F, OutT>), dim3((unsigned)n_tiles), dim3(SCAN_BLOCK), 0, st, f,
+                     n, tiles, n_tiles, out);
+  DN_LAUNCH_CHECK();
+  DN_HIP(hipStreamSynchronize(st));
+  dfree(tiles);
+  return 0;
+}
+
+struct KeepMaskF {
+  const int* count;
+  int min_count;
+  __device__ int64_t operator()(int64_t i) const { return count[i] >= min_count ? 1 : 0; }
+};
+struct CountsF {
+  const int* count;
+  __device__ int64_t operator()(int64_t i) const { return count[i]; }
+};
+struct KeptEntryF {
+  const int32_t* colind;
+  const int32_t* table;
+  __device__ int64_t operator()(int64_t e) const { return table[colind[e]] != -1 ? 1 : 0; }
+};
+struct RowChunksF {
+  const int64_t* rowptr;
+  int64_t chunk;
+  __device__ int64_t operator()(int64_t i) const {
+    int64_t len = rowptr[i + 1] - rowptr[i];
+    return (len + chunk - 1) / chunk;
+  }
+};
+struct LongColF {
+  const int64_t* colptr;
+  int64_t limit;
+  __device__ int64_t operator()(int64_t j) const {
+    return (colptr[j + 1] - colptr[j]) > limit ? 1 : 0;
+  }
+};
+
+int scan_keep_mask(const int* count, int min_count, int64_t n, int32_t* out) {
+  return exclusive_scan(KeepMaskF{count, min_count}, n, out);
+}
+int scan_counts_i64(const int* count, int64_t n, int64_t* out) {
+  return exclusive_scan(CountsF{count}, n, out);
+}
+int scan_kept_entries(const int32_t* colind, const int32_t* table, int64_t nnz, int64_t* out) {
+  return exclusive_scan(KeptEntryF{colind, table}, nnz, out);
+}
+int scan_row_chunks(const int64_t* rowptr, int64_t chunk, int64_t n, int64_t* out) {
+  return exclusive_scan(RowChunksF{rowptr, chunk}, n, out);
+}
+int scan_long_cols(const int64_t* colptr, int64_t limit, int64_t n, int32_t* out) {
+  return exclusive_scan(LongColF{colptr, limit}, n, out);
+}
+
+// ---------------------------------------------------------------------------
+// Loader kernels
+// ---------------------------------------------------------------------------
+
+__global__ void k_pef_rowptr(int64_t n_rows, int64_t k, int64_t* rowptr) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i <= n_rows) rowptr[i] = i * k;
+}
+
+// vals[e] /= (norms[row] + eps); one workgroup walks one row at a time.
+__global__ void __launch_bounds__(256) k_normalize_rows(const int64_t* __restrict__ rowptr,
+                                                        float* __restrict__ vals,
+                                                        const float* __restrict__ norms, float eps,
+                                                        int64_t n_rows) {
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    const float d = norms[row] + eps;
+    const int64_t e1 = rowptr[row + 1];
+    for (int64_t e = rowptr[row] + threadIdx.x; e < e1; e += 256) vals[e] = vals[e] / d;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    k_col_hist(const int32_t* __restrict__ colind, int64_t nnz, int* __restrict__ count) {
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride)
+    atomicAdd(&count[colind[e]], 1);
+}
+
+// og_to_new[i] = pos[i] if kept else -1; new_to_og[pos[i]] = i.
+__global__ void __launch_bounds__(256)
+    k_build_maps(const int* __restrict__ count, int min_count, const int32_t* __restrict__ pos,
+                 int64_t n_cols, int32_t* __restrict__ og_to_new, int32_t* __restrict__ new_to_og) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_cols) return;
+  if (count[i] >= min_count) {
+    og_to_new[i] = pos[i];
+    new_to_og[pos[i]] = (int32_t)i;
+  } else {
+    og_to_new[i] = -1;
+  }
+}
+
+__global__ void __launch_bounds__(256) k_fill_i32(int32_t* p, int64_t n, int32_t v) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// old_to_new[kept[i]] = i; for a column listed twice the last position wins,
+// as in the reference's sequential loop.
+__global__ void __launch_bounds__(256)
+    k_retain_table(const int32_t* __restrict__ kept, int64_t n_kept, int32_t* __restrict__ table) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n_kept) atomicMax(&table[kept[i]], (int32_t)i);
+}
+
+__global__ void __launch_bounds__(256)
+    k_remap_cols(int32_t* __restrict__ colind, int64_t nnz, const int32_t* __restrict__ table) {
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride)
+    colind[e] = table[colind[e]];
+}
+
+// Order-preserving removal of entries whose column was dropped.
+__global__ void __launch_bounds__(256)
+    k_compact_entries(const int32_t* __restrict__ colind, const float* __restrict__ vals,
+                      int64_t nnz, const int32_t* __restrict__ table,
+                      const int64_t* __restrict__ newpos, int32_t* __restrict__ out_col,
+                      float* __restrict__ out_val) {
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride) {
+    int32_t c = table[colind[e]];
+    if (c != -1) {
+      int64_t p = newpos[e];
+      out_col[p] = c;
+      out_val[p] = vals[e];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    k_remap_rowptr(int64_t* __restrict__ rowptr, int64_t n_rows, const int64_t* __restrict__ newpos) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i <= n_rows) rowptr[i] = newpos[rowptr[i]];
+}
+
+// One row of the stable transposition: entry e of this row goes to the next
+// free slot of its column.  Rows are issued in ascending order on one stream
+// and a row holds each column at most once, so every column ends up in
+// ascending row order.
+__global__ void __launch_bounds__(256)
+    k_transpose_row(int32_t row, int64_t e0, int64_t e1, const int32_t* __restrict__ colind,
+                    const float* __restrict__ vals, const int64_t* __restrict__ colptr,
+                    int* __restrict__ cursor, int32_t* __restrict__ rowind,
+                    float* __restrict__ tvals) {
+  int64_t e = e0 + (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= e1) return;
+  int32_t j = colind[e];
+  int64_t p = colptr[j] + atomicAdd(&cursor[j], 1);
+  rowind[p] = row;
+  tvals[p] = vals[e];
+}
+
+__global__ void __launch_bounds__(256)
+    k_collect_long(const int64_t* __restrict__ colptr, int64_t limit, int64_t n_cols,
+                   const int32_t* __restrict__ pos, int32_t* __restrict__ long_cols) {
+  int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (j >= n_cols) return;
+  if (colptr[j + 1] - colptr[j] > limit) long_cols[pos[j]] = (int32_t)j;
+}
+
+__global__ void __launch_bounds__(256)
+    k_sq_norm_partial(const float* __restrict__ v, int64_t n, double* __restrict__ partials) {
+  __shared__ double sh[256];
+  double s = 0.0;
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    double x = (double)v[i];
+    s += x * x;
+  }
+  sh[threadIdx.x] = s;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if (threadIdx.x < off) sh[threadIdx.x] += sh[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partials[blockIdx.x] = sh[0];
+}
+
+static unsigned grid_for(int64_t n, int64_t cap = 1 << 20) {
+  int64_t g = ceil_div(n, 256);
+  if (g < 1) g = 1;
+  if (g > cap) g = cap;
+  return (unsigned)g;
+}
+
+// Drops entries whose table[col] == -1 and renumbers the rest (in place on A).
+static int apply_column_table(dnpeff_csr* A, const int32_t* table, int64_t new_n_cols) {
+  hipStream_t st = stream();
+  int64_t* newpos = nullptr;
+  DN_TRY(dmalloc(&newpos, A->nnz + 1));
+  DN_TRY(scan_kept_entries(A->colind, table, A->nnz, newpos));
+  int64_t new_nnz = 0;
+  DN_HIP(hipMemcpy(&new_nnz, newpos + A->nnz, sizeof(int64_t), hipMemcpyDeviceToHost));
+  if (new_nnz == A->nnz) {
+    hipLaunchKernelGGL(k_remap_cols, dim3(grid_for(A->nnz)), dim3(256), 0, st, A->colind, A->nnz,
+                       table);
+    DN_LAUNCH_CHECK();
+  } else {
+    int32_t* out_col = nullptr;
+    float* out_val = nullptr;
+    DN_TRY(dmalloc(&out_col, new_nnz));
+    DN_TRY(dmalloc(&out_val, new_nnz));
+    hipLaunchKernelGGL(k_compact_entries, dim3(grid_for(A->nnz)), dim3(256), 0, st, A->colind,
+                       A->vals, A->nnz, table, newpos, out_col, out_val);
+    hipLaunchKernelGGL(k_remap_rowptr, dim3(grid_for(A->n_rows + 1)), dim3(256), 0, st, A->rowptr,
+                       A->n_rows, newpos);
+    DN_LAUNCH_CHECK();
+    DN_HIP(hipStreamSynchronize(st));
+    dfree(A->colind);
+    dfree(A->vals);
+    A->colind = out_col;
+    A->vals = out_val;
+    A->nnz = new_nnz;
+  }
+  DN_HIP(hipStreamSynchronize(st));
+  dfree(newpos);
+  A->n_cols = new_n_cols;
+  return 0;
+}
+
+static void drop_derived(dnpeff_csr* A) {
+  dfree(A->colptr); A->colptr = nullptr;
+  dfree(A->rowind); A->rowind = nullptr;
+  dfree(A->tvals); A->tvals = nullptr;
+  dfree(A->chunk_base); A->chunk_base = nullptr; A->n_chunks = 0;
+  dfree(A->long_cols); A->long_cols = nullptr; A->n_long = 0;
+  dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
+}
+
+int csr_ensure_chunks(dnpeff_csr* A) {
+  if (A->chunk_base) return 0;
+  DN_CHECK(A->rowptr != nullptr, "row-major copy of the matrix was released");
+  DN_TRY(dmalloc(&A->chunk_base, A->n_rows + 1));
+  DN_TRY(scan_row_chunks(A->rowptr, SPMM_N_CHUNK, A->n_rows, A->chunk_base));
+  DN_HIP(hipMemcpy(&A->n_chunks, A->chunk_base + A->n_rows, sizeof(int64_t),
+                   hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int csr_ensure_partials(dnpeff_csr* A, int r) {
+  DN_TRY(csr_ensure_chunks(A));
+  int64_t need = A->n_chunks * (int64_t)r;
+  if (need <= A->partials_floats && A->partials) return 0;
+  dfree(A->partials);
+  A->partials = nullptr;
+  DN_TRY(dmalloc(&A->partials, need));
+  A->partials_floats = need;
+  return 0;
+}
+
+}  // namespace dn
+
+using namespace dn;
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+
+DN_API const char* dnpeff_last_error(void) { return g_error; }
+
+DN_API int dnpeff_device_count(int* count) {
+  DN_CHECK(count != nullptr, "count is NULL");
+  int c = 0;
+  hipError_t e = hipGetDeviceCount(&c);
+  if (e != hipSuccess) c = 0;
+  *count = c;
+  return 0;
+}
+
+DN_API int dnpeff_device_info(char* name, int name_len, int64_t* total_bytes, int* n_cus_out) {
+  hipDeviceProp_t p;
+  DN_HIP(hipGetDeviceProperties(&p, 0));
+  if (name && name_len > 0) {
+    strncpy(name, p.name, (size_t)name_len - 1);
+    name[name_len - 1] = 0;
+  }
+  if (total_bytes) *total_bytes = (int64_t)p.totalGlobalMem;
+  if (n_cus_out) *n_cus_out = p.multiProcessorCount;
+  return 0;
+}
+
+DN_API int dnpeff_sync(void) {
+  DN_HIP(hipStreamSynchronize(stream()));
+  return 0;
+}
+
+DN_API void* dnpeff_stream(void) { return (void*)stream(); }
+
+DN_API int dnpeff_dev_malloc(int64_t bytes, void** out) {
+  clear_error();
+  DN_CHECK(out != nullptr && bytes >= 0, "bad arguments");
+  char* p = nullptr;
+  DN_TRY(dmalloc(&p, bytes));
+  *out = p;
+  return 0;
+}
+
+DN_API int dnpeff_dev_free(void* p) {
+  if (!p) return 0;
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipFree(p));
+  return 0;
+}
+
+DN_API int dnpeff_dev_upload(void* dst_dev, const void* src_host, int64_t bytes) {
+  clear_error();
+  DN_CHECK(bytes >= 0 && (bytes == 0 || (dst_dev && src_host)), "bad arguments");
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (bytes) DN_HIP(hipMemcpy(dst_dev, src_host, (size_t)bytes, hipMemcpyHostToDevice));
+  return 0;
+}
+
+DN_API int dnpeff_dev_download(void* dst_host, const void* src_dev, int64_t bytes) {
+  clear_error();
+  DN_CHECK(bytes >= 0 && (bytes == 0 || (dst_host && src_dev)), "bad arguments");
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (bytes) DN_HIP(hipMemcpy(dst_host, src_dev, (size_t)bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+DN_API int64_t dnpeff_size_of_split(int64_t total, int64_t n_splits, int64_t split_index) {
+  if (n_splits <= 0 || split_index < 0 || split_index >= n_splits) return -1;
+  int64_t base = total / n_splits;
+  return split_index == n_splits - 1 ? base + total % n_splits : base;
+}
+
+static int validate_host_csr(int64_t n_rows, int64_t n_cols, int64_t nnz, const int64_t* rowptr) {
+  DN_CHECK(n_rows >= 0 && n_cols >= 0 && nnz >= 0, "negative matrix dimension");
+  DN_CHECK(n_rows < (int64_t)INT32_MAX && n_cols < (int64_t)INT32_MAX,
+           "n_rows and n_cols must fit 32-bit ids");
+  DN_CHECK(rowptr != nullptr, "rowptr is NULL");
+  DN_CHECK(rowptr[0] == 0 && rowptr[n_rows] == nnz, "rowptr[0] must be 0 and rowptr[n_rows] == nnz");
+  for (int64_t i = 0; i < n_rows; i++)
+    DN_CHECK(rowptr[i] <= rowptr[i + 1], "rowptr decreases at row %lld", (long long)i);
+  return 0;
+}
+
+__global__ void __launch_bounds__(256)
+    k_check_cols(const int32_t* __restrict__ colind, int64_t nnz, int64_t n_cols, int* bad) {
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride) {
+    int32_t c = colind[e];
+    if (c < 0 || c >= n_cols) atomicAdd(bad, 1);
+  }
+}
+
+static int check_cols_in_range(const dnpeff_csr* A) {
+  int* bad = nullptr;
+  DN_TRY(dmalloc(&bad, 1));
+  DN_HIP(hipMemsetAsync(bad, 0, sizeof(int), stream()));
+  hipLaunchKernelGGL(k_check_cols, dim3(grid_for(A->nnz)), dim3(256), 0, stream(), A->colind,
+                     A->nnz, A->n_cols, bad);
+  DN_LAUNCH_CHECK();
+  int h = 0;
+  DN_HIP(hipMemcpy(&h, bad, sizeof(int), hipMemcpyDeviceToHost));
+  dfree(bad);
+  DN_CHECK(h == 0, "%d column ids outside [0, n_cols)", h);
+  return 0;
+}
+
+DN_API int dnpeff_csr_from_host(int64_t n_rows, int64_t n_cols, int64_t nnz, const int64_t* rowptr,
+                                const int32_t* colind, const float* vals, dnpeff_csr** out) {
+  clear_error();
+  DN_CHECK(out != nullptr, "out is NULL");
+  *out = nullptr;
+  DN_TRY(validate_host_csr(n_rows, n_cols, nnz, rowptr));
+  DN_CHECK(nnz == 0 || (colind && vals), "colind/vals are NULL");
+  dnpeff_csr* A = new dnpeff_csr();
+  A->n_rows = n_rows; A->n_cols = n_cols; A->nnz = nnz; A->full_dense_size = n_cols;
+  int s = dmalloc(&A->rowptr, n_rows + 1) || dmalloc(&A->colind, nnz) || dmalloc(&A->vals, nnz);
+  if (s) { dnpeff_csr_destroy(A); return 1; }
+  hipError_t e = hipMemcpy(A->rowptr, rowptr, sizeof(int64_t) * (n_rows + 1), hipMemcpyHostToDevice);
+  if (e == hipSuccess && nnz)
+    e = hipMemcpy(A->colind, colind, sizeof(int32_t) * nnz, hipMemcpyHostToDevice);
+  if (e == hipSuccess && nnz)
+    e = hipMemcpy(A->vals, vals, sizeof(float) * nnz, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    set_error("upload of the CSR arrays failed: %s", hipGetErrorString(e));
+    dnpeff_csr_destroy(A);
+    return 1;
+  }
+  if (check_cols_in_range(A)) { dnpeff_csr_destroy(A); return 2; }
+  *out = A;
+  return 0;
+}
+
+DN_API int dnpeff_csr_from_pef(int64_t n_rows, int64_t k, int64_t dense_fisher_size,
+                               const int32_t* indices, const float* values, dnpeff_csr** out) {
+  clear_error();
+  DN_CHECK(out != nullptr, "out is NULL");
+  *out = nullptr;
+  DN_CHECK(n_rows >= 0 && k >= 0 && dense_fisher_size >= 0, "negative dimension");
+  DN_CHECK(n_rows < (int64_t)INT32_MAX && dense_fisher_size < (int64_t)INT32_MAX,
+           "n_rows and dense_fisher_size must fit 32-bit ids");
+  int64_t nnz = n_rows * k;
+  DN_CHECK(nnz == 0 || (indices && values), "indices/values are NULL");
+  dnpeff_csr* A = new dnpeff_csr();
+  A->n_rows = n_rows; A->n_cols = dense_fisher_size; A->nnz = nnz;
+  A->full_dense_size = dense_fisher_size;
+  int s = dmalloc(&A->rowptr, n_rows + 1) || dmalloc(&A->colind, nnz) || dmalloc(&A->vals, nnz);
+  if (s) { dnpeff_csr_destroy(A); return 1; }
+  hipLaunchKernelGGL(k_pef_rowptr, dim3(grid_for(n_rows + 1)), dim3(256), 0, stream(), n_rows, k,
+                     A->rowptr);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && nnz)
+    e = hipMemcpy(A->colind, indices, sizeof(int32_t) * nnz, hipMemcpyHostToDevice);
+  if (e == hipSuccess && nnz)
+    e = hipMemcpy(A->vals, values, sizeof(float) * nnz, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream());
+  if (e != hipSuccess) {
+    set_error("upload of the PEF arrays failed: %s", hipGetErrorString(e));
+    dnpeff_csr_destroy(A);
+    return 1;
+  }
+  if (check_cols_in_range(A)) { dnpeff_csr_destroy(A); return 2; }
+  *out = A;
+  return 0;
+}
+
+DN_API int dnpeff_csr_normalize_rows(dnpeff_csr* A, const float* norms_host, float eps) {
+  clear_error();
+  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(norms_host != nullptr || A->n_rows == 0, "norms is NULL");
+  if (A->n_rows == 0) return 0;
+  float* norms = nullptr;
+  DN_TRY(dmalloc(&norms, A->n_rows));
+  DN_HIP(hipMemcpy(norms, norms_host, sizeof(float) * A->n_rows, hipMemcpyHostToDevice));
+  unsigned grid = (unsigned)(A->n_rows < 65536 ? A->n_rows : 65536);
+  hipLaunchKernelGGL(k_normalize_rows, dim3(grid), dim3(256), 0, stream(), A->rowptr, A->vals,
+                     norms, eps, A->n_rows);
+  DN_LAUNCH_CHECK();
+  DN_HIP(hipStreamSynchronize(stream()));
+  dfree(norms);
+  drop_derived(A);
+  return 0;
+}
+
+DN_API int dnpeff_csr_compact_columns(dnpeff_csr* A, int min_count) {
+  clear_error();
+  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  hipStream_t st = stream();
+  drop_derived(A);
+  const int64_t m_full = A->n_cols;
+  int* count = nullptr;
+  int32_t *pos = nullptr, *og_to_new = nullptr, *new_to_og = nullptr;
+  DN_TRY(dmalloc(&count, m_full));
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m_full > 0 ? m_full : 1), st));
+  hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
+                     count);
+  DN_LAUNCH_CHECK();
+  DN_TRY(dmalloc(&pos, m_full + 1));
+  DN_TRY(scan_keep_mask(count, min_count, m_full, pos));
+  int32_t m_new = 0;
+  DN_HIP(hipMemcpy(&m_new, pos + m_full, sizeof(int32_t), hipMemcpyDeviceToHost));
+  DN_TRY(dmalloc(&og_to_new, m_full));
+  DN_TRY(dmalloc(&new_to_og, (int64_t)m_new));
+  hipLaunchKernelGGL(k_build_maps, dim3(grid_for(m_full)), dim3(256), 0, st, count, min_count, pos,
+                     m_full, og_to_new, new_to_og);
+  DN_LAUNCH_CHECK();
+  DN_HIP(hipStreamSynchronize(st));
+  dfree(count);
+  dfree(pos);
+  A->full_dense_size = m_full;
+  int s = apply_column_table(A, og_to_new, (int64_t)m_new);
+  dfree(og_to_new);
+  if (s) { dfree(new_to_og); return s; }
+  dfree(A->kept);
+  A->kept = new_to_og;
+  return 0;
+}
+
+DN_API int dnpeff_csr_retain_columns(dnpeff_csr* A, const int32_t* kept, int64_t n_kept) {
+  clear_error();
+  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(n_kept >= 0 && (kept || n_kept == 0), "kept is NULL");
+  for (int64_t i = 0; i < n_kept; i++)
+    DN_CHECK(kept[i] >= 0 && kept[i] < A->n_cols, "kept[%lld] = %d outside [0, %lld)",
+             (long long)i, kept[i], (long long)A->n_cols);
+  hipStream_t st = stream();
+  drop_derived(A);
+  int32_t *table = nullptr, *kept_dev = nullptr;
+  DN_TRY(dmalloc(&table, A->n_cols));
+  DN_TRY(dmalloc(&kept_dev, n_kept));
+  if (n_kept) DN_HIP(hipMemcpy(kept_dev, kept, sizeof(int32_t) * n_kept, hipMemcpyHostToDevice));
+  hipLaunchKernelGGL(k_fill_i32, dim3(grid_for(A->n_cols)), dim3(256), 0, st, table, A->n_cols, -1);
+  hipLaunchKernelGGL(k_retain_table, dim3(grid_for(n_kept)), dim3(256), 0, st, kept_dev, n_kept,
+                     table);
+  DN_LAUNCH_CHECK();
+  A->full_dense_size = A->n_cols;
+  int s = apply_column_table(A, table, n_kept);
+  dfree(table);
+  if (s) { dfree(kept_dev); return s; }
+  dfree(A->kept);
+  A->kept = kept_dev;
+  return 0;
+}
+
+DN_API int dnpeff_csr_shape(const dnpeff_csr* A, int64_t* n_rows, int64_t* n_cols, int64_t* nnz) {
+  DN_CHECK(A != nullptr, "matrix is NULL");
+  if (n_rows) *n_rows = A->n_rows;
+  if (n_cols) *n_cols = A->n_cols;
+  if (nnz) *nnz = A->nnz;
+  return 0;
+}
+
+DN_API int dnpeff_csr_full_dense_size(const dnpeff_csr* A, int64_t* out) {
+  DN_CHECK(A && out, "NULL argument");
+  *out = A->full_dense_size;
+  return 0;
+}
+
+DN_API int dnpeff_csr_download(const dnpeff_csr* A, int64_t* rowptr, int32_t* colind, float* vals) {
+  clear_error();
+  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (rowptr)
+    DN_HIP(hipMemcpy(rowptr, A->rowptr, sizeof(int64_t) * (A->n_rows + 1), hipMemcpyDeviceToHost));
+  if (colind && A->nnz)
+    DN_HIP(hipMemcpy(colind, A->colind, sizeof(int32_t) * A->nnz, hipMemcpyDeviceToHost));
+  if (vals && A->nnz)
+    DN_HIP(hipMemcpy(vals, A->vals, sizeof(float) * A->nnz, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+DN_API int dnpeff_csr_kept_indices(const dnpeff_csr* A, int32_t* new_to_og) {
+  clear_error();
+  DN_CHECK(A && new_to_og, "NULL argument");
+  if (A->kept) {
+    if (A->n_cols)
+      DN_HIP(hipMemcpy(new_to_og, A->kept, sizeof(int32_t) * A->n_cols, hipMemcpyDeviceToHost));
+  } else {
+    for (int64_t i = 0; i < A->n_cols; i++) new_to_og[i] = (int32_t)i;
+  }
+  return 0;
+}
+
+DN_API int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out) {
+  clear_error();
+  DN_CHECK(A && out, "NULL argument");
+  const float* v = A->vals ? A->vals : A->tvals;
+  DN_CHECK(v != nullptr || A->nnz == 0, "both copies of the matrix were released");
+  const int blocks = 1024;
+  double* partials = nullptr;
+  DN_TRY(dmalloc(&partials, blocks));
+  hipLaunchKernelGGL(k_sq_norm_partial, dim3(blocks), dim3(256), 0, stream(), v, A->nnz, partials);
+  DN_LAUNCH_CHECK();
+  std::vector<double> h(blocks);
+  DN_HIP(hipMemcpy(h.data(), partials, sizeof(double) * blocks, hipMemcpyDeviceToHost));
+  dfree(partials);
+  double s = 0.0;
+  for (int i = 0; i < blocks; i++) s += h[i];
+  *out = s;
+  return 0;
+}
+
+DN_API int dnpeff_csr_build_transpose(dnpeff_csr* A) {
+  clear_error();
+  DN_CHECK(A != nullptr, "matrix is NULL");
+  if (A->colptr) return 0;
+  DN_CHECK(A->rowptr != nullptr, "row-major copy of the matrix was released");
+  hipStream_t st = stream();
+  const int64_t m = A->n_cols;
+  int* count = nullptr;
+  DN_TRY(dmalloc(&count, m));
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m > 0 ? m : 1), st));
+  hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
+                     count);
+  DN_LAUNCH_CHECK();
+  DN_TRY(dmalloc(&A->colptr, m + 1));
+  DN_TRY(scan_counts_i64(count, m, A->colptr));
+  DN_TRY(dmalloc(&A->rowind, A->nnz));
+  DN_TRY(dmalloc(&A->tvals, A->nnz));
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m > 0 ? m : 1), st));
+  std::vector<int64_t> rowptr((size_t)A->n_rows + 1);
+  DN_HIP(hipMemcpy(rowptr.data(), A->rowptr, sizeof(int64_t) * (A->n_rows + 1),
+                   hipMemcpyDeviceToHost));
+  for (int64_t i = 0; i < A->n_rows; i++) {
+    int64_t len = rowptr[i + 1] - rowptr[i];
+    if (len <= 0) continue;
+    hipLaunchKernelGGL(k_transpose_row, dim3((unsigned)ceil_div(len, 256)), dim3(256), 0, st,
+                       (int32_t)i, rowptr[i], rowptr[i + 1], A->colind, A->vals, A->colptr, count,
+                       A->rowind, A->tvals);
+  }
+  DN_LAUNCH_CHECK();
+  DN_HIP(hipStreamSynchronize(st));
+  dfree(count);
+  // list of long columns for A^T W
+  int32_t* pos = nullptr;
+  DN_TRY(dmalloc(&pos, m + 1));
+  DN_TRY(scan_long_cols(A->colptr, SPMM_T_LONG, m, pos));
+  int32_t n_long = 0;
+  DN_HIP(hipMemcpy(&n_long, pos + m, sizeof(int32_t), hipMemcpyDeviceToHost));
+  A->n_long = n_long;
+  DN_TRY(dmalloc(&A->long_cols, (int64_t)n_long));
+  if (n_long) {
+    hipLaunchKernelGGL(k_collect_long, dim3(grid_for(m)), dim3(256), 0, st, A->colptr, SPMM_T_LONG,
+                       m, pos, A->long_cols);
+    DN_LAUNCH_CHECK();
+  }
+  DN_HIP(hipStreamSynchronize(st));
+  dfree(pos);
+  return 0;
+}
+
+DN_API int dnpeff_csr_download_transpose(dnpeff_csr* A, int64_t* colptr, int32_t* rowind,
+                                         float* vals) {
+  clear_error();
+  DN_TRY(dnpeff_csr_build_transpose(A));
+  if (colptr)
+    DN_HIP(hipMemcpy(colptr, A->colptr, sizeof(int64_t) * (A->n_cols + 1), hipMemcpyDeviceToHost));
+  if (rowind && A->nnz)
+    DN_HIP(hipMemcpy(rowind, A->rowind, sizeof(int32_t) * A->nnz, hipMemcpyDeviceToHost));
+  if (vals && A->nnz)
+    DN_HIP(hipMemcpy(vals, A->tvals, sizeof(float) * A->nnz, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+DN_API int dnpeff_csr_release(dnpeff_csr* A, int which) {
+  clear_error();
+  DN_CHECK(A != nullptr, "matrix is NULL");
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (which == 1) {
+    dfree(A->colind); A->colind = nullptr;
+    dfree(A->vals); A->vals = nullptr;
+    dfree(A->rowptr); A->rowptr = nullptr;
+    dfree(A->chunk_base); A->chunk_base = nullptr; A->n_chunks = 0;
+    dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
+  } else if (which == 2) {
+    dfree(A->colptr); A->colptr = nullptr;
+    dfree(A->rowind); A->rowind = nullptr;
+    dfree(A->tvals); A->tvals = nullptr;
+    dfree(A->long_cols); A->long_cols = nullptr; A->n_long = 0;
+  } else {
+    DN_CHECK(false, "which must be 1 (row-major copy) or 2 (transposed copy)");
+  }
+  return 0;
+}
+
+DN_API int dnpeff_csr_destroy(dnpeff_csr* A) {
+  if (!A) return 0;
+  (void)hipStreamSynchronize(stream());
+  drop_derived(A);
+  dfree(A->rowptr);
+  dfree(A->colind);
+  dfree(A->vals);
+  dfree(A->kept);
+  delete A;
+  return 0;
+}

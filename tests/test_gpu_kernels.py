@@ -1,0 +1,140 @@
+"""Each HIP kernel through its own C-ABI entry point vs the fp64 CPU oracle.
+
+Tolerances: the kernels compute in fp32 with fp32 (MFMA / FMA) accumulation over blocked
+partial sums; against fp64 the bound used is 2e-5 relative to the largest magnitude of the
+output (norm-wise), far inside the 1e-4 the full 50-iteration run has to meet."""
+
+import numpy as np
+import pytest
+
+import npeff_ref_amd as d
+from conftest import random_csr
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-5
+
+
+def _rel(a, b):
+    return np.abs(a.astype(np.float64) - b).max() / max(np.abs(b).max(), 1e-300)
+
+
+def test_mu_bit_exact():
+    rng = np.random.default_rng(0)
+    n = 100003
+    F, num, den = (rng.random(n).astype(np.float32) for _ in range(3))
+    eps = np.float32(1e-8)
+    dF, dn, dd = d.DeviceArray.from_numpy(F), d.DeviceArray.from_numpy(num), d.DeviceArray.from_numpy(den)
+    d.op_mu(dF, dn, dd, eps)
+    want = (F * (num / (den + eps))).astype(np.float32)  # divide first, then multiply
+    assert np.array_equal(dF.numpy(), want)
+
+
+@pytest.mark.parametrize("r", [16, 50, 64, 128, 256, 512])
+@pytest.mark.parametrize("shape", [(37, 900, 60), (130, 5000, 3000)])
+def test_spmm_n_and_t(r, shape):
+    n, m, maxk = shape
+    rng = np.random.default_rng(r + n)
+    rp, ci, va = random_csr(rng, n, m, maxk, empty_rows={1, n - 1})
+    A = d.Csr.from_host(rp, ci, va, m)
+    H = rng.random((m, r)).astype(np.float32)
+    W = rng.random((n, r)).astype(np.float32)
+    dH, dW = d.DeviceArray.from_numpy(H), d.DeviceArray.from_numpy(W)
+    dN, dT = d.DeviceArray((n, r)), d.DeviceArray((m, r))
+    d.op_spmm_n(A, r, dH, dN)
+    d.op_spmm_t(A, r, dW, dT)
+    N, T = dN.numpy(), dT.numpy()
+    assert _rel(N, orc.spmm_n_f64(rp, ci, va, H)) < TOL
+    assert _rel(T, orc.spmm_t_f64(rp, ci, va, m, W)) < TOL
+    assert np.all(N[1] == 0) and np.all(N[n - 1] == 0)  # empty rows
+    # reproducible bit for bit
+    d.op_spmm_n(A, r, dH, dN)
+    d.op_spmm_t(A, r, dW, dT)
+    assert np.array_equal(dN.numpy(), N) and np.array_equal(dT.numpy(), T)
+    A.close()
+
+
+def test_spmm_long_rows_and_long_columns():
+    """Rows spanning several work chunks and columns long enough for the workgroup path."""
+    rng = np.random.default_rng(5)
+    n, m, r = 700, 20000, 128
+    rowptr, colind, vals, _ = d.synth_pef_host(n, m, k_fixed=5000, zipf_s=1.1, seed=2)
+    A = d.Csr.from_host(rowptr, colind, vals, m)
+    H = rng.random((m, r)).astype(np.float32)
+    W = rng.random((n, r)).astype(np.float32)
+    dN, dT = d.DeviceArray((n, r)), d.DeviceArray((m, r))
+    d.op_spmm_n(A, r, d.DeviceArray.from_numpy(H), dN)
+    d.op_spmm_t(A, r, d.DeviceArray.from_numpy(W), dT)
+    assert _rel(dN.numpy(), orc.spmm_n_f64(rowptr, colind, vals, H)) < TOL
+    assert _rel(dT.numpy(), orc.spmm_t_f64(rowptr, colind, vals, m, W)) < TOL
+    A.close()
+
+
+@pytest.mark.parametrize("rows,r", [(1, 16), (31, 16), (1000, 50), (4097, 128), (20000, 256), (9000, 512), (300, 130)])
+def test_gram(rows, r):
+    rng = np.random.default_rng(rows + r)
+    X = rng.random((rows, r)).astype(np.float32)
+    dG = d.DeviceArray((r, r))
+    d.op_gram(d.DeviceArray.from_numpy(X), dG)
+    G = dG.numpy()
+    want = orc.gram_f64(X)
+    assert _rel(G, want) < TOL
+    assert np.array_equal(G, G.T) or _rel(G, G.T.astype(np.float64)) < 1e-6
+
+
+@pytest.mark.parametrize("rows,r", [(1, 16), (33, 16), (1000, 50), (4100, 128), (5000, 256), (3000, 512), (300, 130)])
+def test_xg_mu(rows, r):
+    rng = np.random.default_rng(rows * 3 + r)
+    X = rng.random((rows, r)).astype(np.float32)
+    G = rng.random((r, r)).astype(np.float32)  # deliberately not symmetric
+    num = rng.random((rows, r)).astype(np.float32)
+    eps = np.float32(1e-8)
+    dX, dG, dnum = d.DeviceArray.from_numpy(X), d.DeviceArray.from_numpy(G), d.DeviceArray.from_numpy(num)
+    dout, dD = d.DeviceArray((rows, r)), d.DeviceArray((rows, r))
+    d.op_xg_mu(dX, dG, dnum, eps, dout, dD)
+    want, wantD = orc.xg_mu_f64(X, G, num, eps)
+    assert _rel(dD.numpy(), wantD) < TOL
+    assert _rel(dout.numpy(), want) < TOL
+    # in place on the numerator buffer gives the same bits
+    out1 = dout.numpy()
+    d.op_xg_mu(dX, dG, dnum, eps, dnum, None)
+    assert np.array_equal(dnum.numpy(), out1)
+
+
+def test_dot_fp64_accumulation():
+    rng = np.random.default_rng(1)
+    n = 3_000_001
+    x, y = rng.random(n).astype(np.float32), rng.random(n).astype(np.float32)
+    got = d.op_dot(d.DeviceArray.from_numpy(x), d.DeviceArray.from_numpy(y))
+    want = np.dot(x.astype(np.float64), y.astype(np.float64))
+    assert abs(got - want) / want < 1e-13
+
+
+def test_init_uniform_matches_host_rule():
+    seed, n, r, m = 43190432042, 37, 16, 211
+    dW, dH = d.DeviceArray((n, r)), d.DeviceArray((m, r))
+    d.op_init_uniform(0, n, r, seed, dW)
+    d.op_init_uniform(1, r, m, seed, dH)
+    W, Ht = dW.numpy(), dH.numpy()
+    for i, c in [(0, 0), (5, 3), (36, 15)]:
+        assert W[i, c] == np.float32(d.uniform_at(seed, 0, i, c, r))
+    for c, j in [(0, 0), (7, 100), (15, 210)]:
+        assert Ht[j, c] == np.float32(d.uniform_at(seed, 1, c, j, m))
+
+
+@pytest.mark.parametrize("r", [16, 100, 256])
+def test_spsp_dense(r):
+    rng = np.random.default_rng(40 + r)
+    n, m = 150, 6000
+    a = random_csr(rng, n, m, 3000, empty_rows={2})
+    b = random_csr(rng, r, m, 400, sort_cols=True)
+    A, B = d.Csr.from_host(*a, m), d.Csr.from_host(*b, m)
+    out = d.DeviceArray((n, r))
+    d.op_spsp_dense(A, B, out)
+    assert _rel(out.numpy(), orc.spsp_dense_f64(a, m, b, r)) < TOL
+    hh = d.DeviceArray((r, r))
+    d.op_spsp_dense(B, B, hh)
+    assert _rel(hh.numpy(), orc.spsp_dense_f64(b, m, b, r)) < TOL
+    A.close()
+    B.close()
