@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""D-NPEFF NMF benchmark on one MI355X: MU iterations/sec on BASELINE.json configs[1]
+(10,000 examples x 110M features, 65,536 nnz/row, Zipf 1.1 columns, r = 128), per-kernel
+roofline fractions from HIP events, and the same update loop timed on the host cores.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Prints ONE JSON line.  A step is one MU iteration (W-update then H-update) with the CSR
+matrix and the factors already resident in HBM; the loss is not evaluated inside the timed
+region, exactly as the reference's own timer excludes it
+(cc/cuda_d_npeff/src/nmf/sparse/multi_mu_dense_factors_nmf1.h:188-200)."""
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
+MFMA_FP32_PEAK = 157.3e12  # flop/s, dense fp32 matrix
+
+CONFIGS = {
+    "c0": dict(n=512, m_full=1 << 20, k=4096, kmin=0, kmax=0, s=1.1, r=16),
+    "c1": dict(n=10_000, m_full=110_000_000, k=65_536, kmin=0, kmax=0, s=1.1, r=128),
+    "c1-small": dict(n=1_000, m_full=11_000_000, k=16_384, kmin=0, kmax=0, s=1.1, r=128),
+}
+
+
+def log(msg):
+    print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
+
+
+def algorithmic(cls, n, m, z, r):
+    """Compulsory traffic / flops of one launch: every operand touched once."""
+    P = 4 if z < 2**31 else 8
+    if cls == "spmm_n":
+        return "hbm", 8 * z + P * (n + 1) + 4 * r * m + 4 * n * r
+    if cls == "spmm_n_reduce":
+        return "hbm", 8 * n * r
+    if cls == "spmm_t":
+        return "hbm", 8 * z + P * (m + 1) + 4 * n * r + 4 * r * m
+    if cls == "gram_H":
+        return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 4 * m * r + 4 * r * r)
+    if cls == "gram_W":
+        return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 4 * n * r + 4 * r * r)
+    if cls == "xg_mu_H":
+        return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 12 * m * r + 4 * r * r)
+    if cls == "xg_mu_W":
+        return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 12 * n * r + 4 * r * r)
+    raise KeyError(cls)
+
+
+def prepare_cpu_baseline(d, A, nmf, n, m, r, eps):
+    """Copies the CSR matrix and the initial factors to the host for the fp32 OpenMP port of the
+    reference loop (oracle/dnpeff_oracle.c: orc_f32_step)."""
+    from oracle import oracle as orc
+
+    t0 = time.perf_counter()
+    rp, ci, va = A.download()
+    W0 = nmf.loadWToHostSync()
+    Ht0 = np.empty((m, r), dtype=np.float32)
+    wdev, hdev = C.c_void_p(), C.c_void_p()
+    d.binding._check(d.lib.dnpeff_nmf_device_factors(nmf._h, C.byref(wdev), C.byref(hdev)))
+    d.binding._check(d.lib.dnpeff_dev_download(Ht0.ctypes.data_as(C.c_void_p), hdev, Ht0.nbytes))
+    log(f"cpu baseline: inputs on the host in {time.perf_counter() - t0:.1f} s")
+    t0 = time.perf_counter()
+    base = orc.F32Baseline(rp, ci, va, m, W0, eps=eps, Ht0_mr=Ht0)
+    del Ht0
+    log(f"cpu baseline: context (host transposed CSR) in {time.perf_counter() - t0:.1f} s, "
+        f"{orc.F32Baseline.num_threads()} threads")
+    return base
+
+
+def run_cpu_baseline(base, steps, n, m, z, r):
+    from oracle import oracle as orc
+
+    t0 = time.perf_counter()
+    base.step(steps)
+    el = time.perf_counter() - t0
+    base.close()
+    log(f"cpu baseline: {steps} step(s) in {el:.2f} s")
+    return {"value": steps / el, "unit": "MU iterations/s", "cores": orc.F32Baseline.num_threads(),
+            "kind": "port",
+            "sample": f"{steps} full MU iteration(s) of the same workload (n={n}, m={m}, nnz={z}, r={r}), "
+                      "fp32 OpenMP port of the reference loop, loss excluded"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
+    ap.add_argument("--eps", type=float, default=1e-12)
+    ap.add_argument("--seed", type=int, default=43190432042)
+    ap.add_argument("--cpu-steps", type=int, default=1,
+                    help="MU iterations timed on the host cores (0 = skip)")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build drives exactly one GPU (no collectives are built); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import npeff_ref_amd as d
+
+    if d.device_count() < 1:
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    cfg = CONFIGS[args.config]
+    name, hbm_bytes, cus = d.device_info()
+    log(f"device {name}, {hbm_bytes / 2**30:.0f} GiB, {cus} CUs; workload {args.config} {cfg}")
+
+    t0 = time.perf_counter()
+    A, norms = d.Csr.synth(cfg["n"], cfg["m_full"], k_fixed=cfg["k"], k_min=cfg["kmin"],
+                           k_max=cfg["kmax"], zipf_s=cfg["s"], seed=args.seed)
+    log(f"generated {A.nnz} entries on the device in {time.perf_counter() - t0:.1f} s")
+    t0 = time.perf_counter()
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    n, m, z = A.n_rows, A.n_cols, A.nnz
+    log(f"normalised + compacted: n={n} m={m} (of {cfg['m_full']}) nnz={z} "
+        f"in {time.perf_counter() - t0:.1f} s")
+    r = cfg["r"]
+    t0 = time.perf_counter()
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=0, eps=args.eps, seed=args.seed))
+    nmf.initialize()
+    d.sync()
+    log(f"context (transposed CSR, factors) in {time.perf_counter() - t0:.1f} s")
+
+    # the CPU baseline starts from the same factors, so copy them before the GPU loop runs
+    cpu = prepare_cpu_baseline(d, A, nmf, n, m, r, args.eps) if args.cpu_steps > 0 else None
+
+    nmf.step(args.warmup)
+    d.sync()
+    nmf.set_profiling(True)
+    nmf.timings(reset=True)
+    d.sync()
+    t0 = time.perf_counter()
+    nmf.step(args.steps)
+    d.sync()
+    elapsed = time.perf_counter() - t0
+    tim = nmf.timings(reset=True)
+    nmf.set_profiling(False)
+    loss = nmf.computeUncachedLoss()
+    ms_per_step = elapsed * 1e3 / args.steps
+    log(f"{args.steps} steps in {elapsed:.3f} s -> {ms_per_step:.2f} ms/step, loss {loss:.6g}")
+
+    kernels = {}
+    for cls, (ms_sum, cnt) in tim.items():
+        if cnt == 0:
+            continue
+        bound, work = algorithmic(cls, n, m, z, r)
+        avg_s = ms_sum / cnt * 1e-3
+        peak = HBM_PEAK if bound == "hbm" else MFMA_FP32_PEAK
+        kernels[cls] = dict(
+            ms=ms_sum / cnt, bound=bound,
+            achieved=work / avg_s / 1e9 if bound == "hbm" else work / avg_s / 1e12,
+            unit="GB/s" if bound == "hbm" else "TFLOP/s", frac=work / avg_s / peak,
+            share=ms_sum / (elapsed * 1e3))
+        k = kernels[cls]
+        log(f"  {cls:14s} {k['ms']:9.3f} ms  {k['achieved']:9.1f} {k['unit']:8s} frac {k['frac']:.3f}")
+    dom = max((k for k in kernels if k != "spmm_n_reduce"), key=lambda k: kernels[k]["ms"])
+    kd = kernels[dom]
+    roofline = dict(kernel=dom, bound=kd["bound"], achieved=kd["achieved"],
+                    peak=HBM_PEAK / 1e9 if kd["bound"] == "hbm" else MFMA_FP32_PEAK / 1e12,
+                    unit=kd["unit"], frac=kd["frac"], traffic=None)
+
+    cpu_baseline = run_cpu_baseline(cpu, args.cpu_steps, n, m, z, r) if cpu is not None else None
+
+    out = {
+        "metric": "NMF MU iterations/sec + SpMM achieved HBM GB/s (% of peak), 1 MI355X",
+        "value": args.steps / elapsed,
+        "unit": "MU iterations/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1] D-NPEFF NMF" if args.config == "c1" else args.config,
+                   "n_examples": n, "n_features_full": cfg["m_full"], "n_features_kept": m,
+                   "nnz": z, "nnz_per_row": cfg["k"], "zipf_s": cfg["s"], "rank": r,
+                   "eps": args.eps, "seed": args.seed},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "kernels": kernels,
+        "spmm_hbm_frac": {k: kernels[k]["frac"] for k in ("spmm_n", "spmm_t") if k in kernels},
+        "loss_after": loss,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
