@@ -1,0 +1,128 @@
+// run_nmf_on_pefs: reads a D-PEF hdf5 file, normalises the rows, drops sparse columns and runs
+// multiplicative-update NMF with dense W and H on one MI355X through the C ABI of dnpeff.h;
+// writes W, H and the kept-column map.  Flags, order of steps, defaults and stdout lines follow
+// cc/cuda_d_npeff/mains/run_nmf_on_pefs.cu:15-259; the loop and its timer follow
+// cc/cuda_d_npeff/src/nmf/sparse/multi_mu_dense_factors_nmf1.h:152-205.
+#include <chrono>
+#include <climits>
+#include <cmath>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "../../../include/dnpeff.h"
+#include "flags.hpp"
+#include "h5io.hpp"
+
+using hostutil::fatal;
+
+static void ck(int status) {
+  if (status) fatal(std::string("Error: ") + dnpeff_last_error());
+}
+
+struct ProgramFlags {
+  std::string output_path, pef_path;
+  int n_components = 0, max_iters = 0;
+  int n_examples = -1, n_fisher_values = -1;
+  float sparsity_W = -1.0f;            // accepted, without effect (as in the reference)
+  int min_values_per_parameter = 1;
+  std::string initial_H_path, initial_W_path;  // accepted, without effect (as in the reference)
+  // additions (optional): the reference hard-codes these at run_nmf_on_pefs.cu:189-192
+  float eps = 1e-8f;
+  long seed = 43190432042L;
+  int log_every = 10;
+};
+
+static ProgramFlags parse_flags(int argc, char** argv) {
+  hostutil::Flags f(argc, argv);
+  ProgramFlags p;
+  f.read("output_path", &p.output_path);
+  f.read("per_example_fishers", &p.pef_path);
+  f.read("nmf_n_components", &p.n_components);
+  f.read("nmf_max_iter", &p.max_iters);
+  f.read("n_examples", &p.n_examples, false);
+  f.read("n_fisher_values", &p.n_fisher_values, false);
+  f.read("min_values_per_parameter", &p.min_values_per_parameter, false);
+  f.read("sparsity_W", &p.sparsity_W, false);
+  f.read("initial_H_path", &p.initial_H_path, false);
+  f.read("initial_W_path", &p.initial_W_path, false);
+  f.read("eps", &p.eps, false);
+  f.read("seed", &p.seed, false);
+  f.read("log_every", &p.log_every, false);
+  return p;  // unknown flags are ignored, as in the reference
+}
+
+int main(int argc, char** argv) {
+  ProgramFlags flags = parse_flags(argc, argv);
+
+  h5io::PefDims dims = h5io::pef_dims(flags.pef_path, flags.n_examples, flags.n_fisher_values);
+  const long nnz_in = dims.n_rows * dims.n_values_per_row;
+  // Row offsets are always 64-bit and column ids 32-bit here; the line is kept for log parity.
+  if (nnz_in > (long)INT32_MAX)
+    std::cout << "Reading in PEFs using 64 bit indices.\n";
+  else
+    std::cout << "Using 32 bit indices.\n";
+
+  int n_devices = 0;
+  ck(dnpeff_device_count(&n_devices));
+  if (n_devices < 1) fatal("Error: no GPU visible.");
+
+  std::cout << "Starting to read in PEFs.\n";
+  h5io::Pef pef = h5io::read_pef(flags.pef_path, flags.n_examples, flags.n_fisher_values);
+  std::cout << "PEFS read in.\n";
+
+  dnpeff_csr* A = nullptr;
+  ck(dnpeff_csr_from_pef(pef.n_rows, pef.k, pef.dense_fisher_size, pef.indices.data(),
+                         pef.values.data(), &A));
+  pef.values = std::vector<float>();
+  pef.indices = std::vector<int32_t>();
+  ck(dnpeff_csr_normalize_rows(A, pef.norms.data(), 1e-9f));
+
+  int64_t n = 0, m = 0, nnz = 0;
+  ck(dnpeff_csr_shape(A, &n, &m, &nnz));
+  std::cout << "n_cols before reduction: " << m << "\n";
+  ck(dnpeff_csr_compact_columns(A, flags.min_values_per_parameter));
+  ck(dnpeff_csr_shape(A, &n, &m, &nnz));
+  std::cout << "n_cols after reduction: " << m << " [density=" << (double)nnz / (double)(n * m)
+            << "]\n";
+
+  std::cout << "Initializing NMF.\n";
+  dnpeff_nmf* nmf = nullptr;
+  ck(dnpeff_nmf_create(A, flags.n_components, flags.eps, flags.seed, &nmf));
+  ck(dnpeff_nmf_init_factors(nmf));
+  ck(dnpeff_sync());
+
+  std::cout << "Running NMF.\n";
+  auto t_start = std::chrono::high_resolution_clock::now();
+  for (int step = 0; step < flags.max_iters; step++) {
+    ck(dnpeff_nmf_step(nmf, 1));
+    if (flags.log_every > 0 && (step + 1) % flags.log_every == 0) {
+      ck(dnpeff_sync());
+      auto t_end = std::chrono::high_resolution_clock::now();
+      double elapsed_ms = std::chrono::duration<double, std::milli>(t_end - t_start).count();
+      double loss = 0.0;
+      ck(dnpeff_nmf_loss(nmf, &loss));
+      // the ms/step figure ignores the time spent on the loss
+      std::cout << "step " << step + 1 << ": " << (float)loss << " ["
+                << elapsed_ms / (double)flags.log_every << " ms/step]\n";
+      t_start = std::chrono::high_resolution_clock::now();
+    }
+  }
+  ck(dnpeff_sync());
+
+  const int r = flags.n_components;
+  std::vector<float> W((size_t)n * r), H((size_t)r * m);
+  std::vector<int32_t> kept((size_t)m);
+  ck(dnpeff_nmf_get_W(nmf, W.data()));
+  ck(dnpeff_nmf_get_H(nmf, H.data()));
+  ck(dnpeff_csr_kept_indices(A, kept.data()));
+  int64_t full = 0;
+  ck(dnpeff_csr_full_dense_size(A, &full));
+
+  std::cout << "Saving decomposition to file.\n";
+  h5io::write_dense_decomposition(flags.output_path, n, r, m, W.data(), H.data(), kept.data(),
+                                  (int32_t)full);
+  dnpeff_nmf_destroy(nmf);
+  dnpeff_csr_destroy(A);
+  return 0;
+}

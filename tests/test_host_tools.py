@@ -1,0 +1,168 @@
+"""The C++ host executables: flag behaviour and file layouts on the CPU; the full pipelines
+(hdf5 in -> GPU NMF -> hdf5 out) on the GPU, compared with the same fit driven through the
+C ABI from Python."""
+
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import h5lite
+import npeff_ref_amd as d
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "npeff_ref_amd", "bin")
+
+pytestmark = pytest.mark.skipif(
+    not (h5lite.available and os.path.exists(os.path.join(BIN, "run_nmf_on_pefs"))),
+    reason="host executables / HDF5 library not built",
+)
+
+
+def run(prog, *flags, check=False):
+    p = subprocess.run([os.path.join(BIN, prog), *flags], capture_output=True, text=True, timeout=600)
+    if check:
+        assert p.returncode == 0, p.stdout + p.stderr
+    return p
+
+
+def make_pef(tmp_path, n=24, m=20000, k=300, seed=3, **extra):
+    path = str(tmp_path / "pef.h5")
+    flags = [f"--output_path={path}", f"--n_examples={n}", f"--n_parameters={m}", f"--n_fisher_values={k}",
+             f"--seed={seed}"] + [f"--{a}={b}" for a, b in extra.items()]
+    run("synth_pef_h5", *flags, check=True)
+    return path
+
+
+# ---- CPU: flags and schemas -----------------------------------------------------------------
+def test_missing_required_flag_is_fatal(tmp_path):
+    p = run("run_nmf_on_pefs", "--output_path=/tmp/x.h5")
+    assert p.returncode != 0 and "Missing flag: per_example_fishers" in p.stdout
+    p = run("fit_coeffs_to_sparse_H", "--output_path=/tmp/x.h5", "--pef_path=a")
+    assert p.returncode != 0 and "Missing flag: H_path" in p.stdout
+
+
+def test_fit_rejects_unknown_flags_but_nmf_ignores_them(tmp_path):
+    p = run("fit_coeffs_to_sparse_H", "--output_path=o", "--pef_path=a", "--H_path=b", "--n_splits_sparse_matmul=1",
+            "--n_row_splits_pefs=1", "--nmf_max_iter=1", "--bogus=3")
+    assert p.returncode != 0 and "Unrecognized flags." in p.stdout
+
+
+def test_synthetic_pef_file_has_the_reference_schema(tmp_path):
+    path = make_pef(tmp_path, n=10, m=5000, k=64, seed=9)
+    vals, idx = h5lite.read(path, "data/fisher/values"), h5lite.read(path, "data/fisher/indices")
+    norms = h5lite.read(path, "data/dense_fisher_norms")
+    assert vals.dtype == np.float32 and vals.shape == (10, 64)
+    assert idx.dtype == np.int32 and idx.shape == (10, 64)
+    assert norms.dtype == np.float32 and norms.shape == (10,)
+    a, shape = h5lite.attr(path, "data/fisher", "dense_fisher_size")
+    assert a.dtype == np.int32 and a.itemsize == 4 and int(a[0]) == 5000
+    hr, hc, hv, hn = d.synth_pef_host(10, 5000, k_fixed=64, seed=9)
+    assert np.array_equal(idx.ravel(), hc) and np.array_equal(vals.ravel(), hv) and np.array_equal(norms, hn)
+
+
+def test_truncation_flags_larger_than_the_file_are_fatal(tmp_path):
+    path = make_pef(tmp_path, n=4, m=1000, k=16)
+    p = run("run_nmf_on_pefs", f"--output_path={tmp_path}/o.h5", f"--per_example_fishers={path}",
+            "--nmf_n_components=2", "--nmf_max_iter=1", "--n_examples=5")
+    assert p.returncode != 0 and "n_examples exceeds" in p.stdout
+
+
+# ---- GPU: the pipelines ---------------------------------------------------------------------
+@pytest.mark.gpu
+def test_run_nmf_on_pefs_end_to_end(tmp_path):
+    n, m_full, k, r, iters = 40, 30000, 500, 16, 20
+    pef = make_pef(tmp_path, n=n + 8, m=m_full, k=k + 40, seed=11)
+    out = str(tmp_path / "decomp.h5")
+    p = run("run_nmf_on_pefs", f"--output_path={out}", f"--per_example_fishers={pef}", f"--nmf_n_components={r}",
+            f"--nmf_max_iter={iters}", f"--n_examples={n}", f"--n_fisher_values={k}", "--min_values_per_parameter=2",
+            "--sparsity_W=0.5", "--some_unknown_flag=1", check=True)
+    lines = p.stdout.splitlines()
+    assert "Using 32 bit indices." in lines and "PEFS read in." in lines and "Running NMF." in lines
+    assert f"n_cols before reduction: {m_full}" in lines
+    steps = [l for l in lines if l.startswith("step ")]
+    assert [s.split(":")[0] for s in steps] == ["step 10", "step 20"] and all("ms/step]" in s for s in steps)
+
+    # the same fit through the C ABI from Python, with the reference defaults (eps 1e-8, seed)
+    vals = h5lite.read(pef, "data/fisher/values")[:n, :k]
+    idx = h5lite.read(pef, "data/fisher/indices")[:n, :k]
+    norms = h5lite.read(pef, "data/dense_fisher_norms")[:n]
+    A = d.Csr.from_pef(idx, vals, m_full)
+    A.normalize_rows(norms)
+    A.compact_columns(2)
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=iters))
+    hist = nmf.run(log=lambda s: None)
+    W, H, kept = h5lite.read(out, "data/W"), h5lite.read(out, "data/H"), h5lite.read(out, "data/reduce_kept_indices")
+    assert W.dtype == np.float32 and W.shape == (n, r) and H.shape == (r, A.n_cols)
+    assert np.array_equal(W, nmf.loadWToHostSync()) and np.array_equal(H, nmf.loadHToHostSync())
+    assert kept.dtype == np.int32 and np.array_equal(kept, A.kept_indices())
+    fds, shape = h5lite.attr(out, "data/reduce_kept_indices", "full_dense_size")
+    assert shape == (1,) and int(fds[0]) == m_full  # the reference writes shape (1,) here
+    logged = float(steps[-1].split(":")[1].split("[")[0])
+    assert abs(logged - hist[-1][1]) / hist[-1][1] < 1e-5
+    # and against the fp64 oracle
+    rp, ci, va = A.download()
+    W0 = np.array([[d.uniform_at(43190432042, 0, i, c, r) for c in range(r)] for i in range(n)], np.float32)
+    nmf2 = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=0))
+    nmf2.initialize()
+    assert np.array_equal(nmf2.loadWToHostSync(), W0)
+    W64, H64, losses = orc.nmf_f64(rp, ci, va, A.n_cols, W0, nmf2.loadHToHostSync(), np.float32(1e-8), iters, 10)
+    assert np.linalg.norm(W - W64) / np.linalg.norm(W64) < 1e-4
+    assert np.linalg.norm(H - H64) / np.linalg.norm(H64) < 1e-4
+    assert abs(logged - losses[-1]) / losses[-1] < 1e-4
+
+
+@pytest.mark.gpu
+def test_fit_coeffs_to_sparse_H_end_to_end(tmp_path):
+    n, m_full, k, r, iters = 50, 20000, 400, 8, 50
+    pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=21, sparse_H_output_path=str(tmp_path / "H.h5"), rank=r,
+                   H_density=0.02)
+    hpath, out = str(tmp_path / "H.h5"), str(tmp_path / "fit.h5")
+    p = run("fit_coeffs_to_sparse_H", f"--output_path={out}", f"--pef_path={pef}", f"--H_path={hpath}",
+            "--n_splits_sparse_matmul=4", "--n_row_splits_pefs=2", f"--nmf_max_iter={iters}", check=True)
+    lines = p.stdout.splitlines()
+    assert "Finished running first stage." in lines and "Finished running second stage." in lines
+    steps = [l for l in lines if l.startswith("step ")]
+    assert [s.split(":")[0] for s in steps] == ["step 25", "step 50"]
+    # output layout: new W, unchanged sparse H, scalar full_dense_size
+    for name in ("values", "row_indices", "column_indices"):
+        assert np.array_equal(h5lite.read(out, f"data/H/{name}"), h5lite.read(hpath, f"data/H/{name}"))
+    assert h5lite.read(out, "data/H/row_indices").dtype == np.int64
+    shape_attr, _ = h5lite.attr(out, "data/H", "shape")
+    assert shape_attr.tolist() == [r, m_full]
+    fds, shape = h5lite.attr(out, "data/reduce_kept_indices", "full_dense_size")
+    assert shape == () and int(fds[0]) == m_full
+    W = h5lite.read(out, "data/W")
+    assert W.shape == (n, r)
+    # fp64 oracle of both stages on the same inputs
+    vals, idx = h5lite.read(pef, "data/fisher/values"), h5lite.read(pef, "data/fisher/indices")
+    norms = h5lite.read(pef, "data/dense_fisher_norms")
+    rp = orc.pef_rowptr(n, k)
+    va = orc.normalize_rows(rp, vals.ravel(), norms)
+    kept = h5lite.read(hpath, "data/reduce_kept_indices")
+    rp2, ci2, va2 = orc.retain_columns(rp, idx.ravel(), va, m_full, kept)
+    b = (h5lite.read(hpath, "data/H/row_indices"), h5lite.read(hpath, "data/H/column_indices"),
+         h5lite.read(hpath, "data/H/values"))
+    AH = orc.spsp_dense_f64((rp2, ci2, va2), m_full, b, r)
+    HH = orc.spsp_dense_f64(b, m_full, b, r)
+    W0 = np.array([[d.uniform_at(43190432042, 0, i, c, r) for c in range(r)] for i in range(n)], np.float32)
+    W64, ref, tru = orc.fit_f64(AH, HH, float(np.sum(va2.astype(np.float64) ** 2)), W0, np.float32(1e-7), iters, 25)
+    assert np.linalg.norm(W - W64) / np.linalg.norm(W64) < 1e-4
+    logged = [float(s.split(":")[1].split("[")[0]) for s in steps]
+    assert np.all(np.abs(np.array(logged) - ref) / ref < 1e-4)
+
+
+@pytest.mark.gpu
+def test_fit_row_split_check_is_kept(tmp_path):
+    """A split with nnz >= INT32_MAX is fatal in the reference; with small inputs the check passes
+    for any number of splits, including more splits than rows' worth of remainder."""
+    pef = make_pef(tmp_path, n=7, m=3000, k=50, seed=2, sparse_H_output_path=str(tmp_path / "H.h5"), rank=4,
+                   H_density=0.05)
+    p = run("fit_coeffs_to_sparse_H", f"--output_path={tmp_path}/o.h5", f"--pef_path={pef}",
+            f"--H_path={tmp_path}/H.h5", "--n_splits_sparse_matmul=1", "--n_row_splits_pefs=3", "--nmf_max_iter=2",
+            "--DEV_n_cols=1000", check=True)
+    assert "NOTE: Using flag intended only for development purposes." in p.stdout
+    shape_attr, _ = h5lite.attr(f"{tmp_path}/o.h5", "data/H", "shape")
+    assert shape_attr.tolist() == [4, 1000]
