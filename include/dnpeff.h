@@ -304,6 +304,10 @@ int dnpeff_op_dot(int64_t count, const float* x, const float* y, double* out_hos
  * (cc/cuda_d_npeff/src/cuda/ops/spsp_matmul.h:95-131). */
 int dnpeff_op_spsp_dense(dnpeff_csr* A, dnpeff_csr* B, float* out_nr);
 
+/* dst[i] = src[i], i < count: a plain streaming copy of known size, the yardstick
+ * that hardware-counter readings (FETCH_SIZE, WRITE_SIZE) are scaled by. */
+int dnpeff_op_copy(int64_t count, const float* src, float* dst);
+
 /* x[i] = U[0,1) value of logical element i of matrix matrix_id, written in the
  * device layout (see dnpeff_uniform_at). */
 int dnpeff_op_init_uniform(int matrix_id, int64_t logical_rows, int64_t logical_cols,

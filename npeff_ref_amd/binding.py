@@ -99,6 +99,7 @@ SIGNATURES = {
     "dnpeff_op_xg_mu": (C.c_int, [_i64, C.c_int, _p, _p, _p, _f32, _p, _p]),
     "dnpeff_op_dot": (C.c_int, [_i64, _p, _p, C.POINTER(_f64)]),
     "dnpeff_op_spsp_dense": (C.c_int, [_p, _p, _p]),
+    "dnpeff_op_copy": (C.c_int, [_i64, _p, _p]),
     "dnpeff_op_init_uniform": (C.c_int, [C.c_int, _i64, _i64, _u64, _p]),
 }
 

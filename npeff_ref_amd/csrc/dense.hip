@@ -148,7 +148,7 @@ __global__ void __launch_bounds__(256)
 }
 
 int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace) {
-  DN_CHECK(r >= 1 && r <= 4096, "rank %d outside [1, 4096]", r);
+  DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
   int tiles = (int)ceil_div(r, GRAM_TILE);
   int64_t slices = gram_slices(rows);
   int64_t rps = ceil_div(rows > 0 ? rows : 1, slices);
@@ -164,91 +164,193 @@ int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace)
 // ---------------------------------------------------------------------------
 // out = X * num / (X G + eps)
 //
-// A wave owns 32 rows of X and up to 128 output columns (4 MFMA blocks); the
-// workgroup's 4 waves own 128 consecutive rows.  The contraction runs over the
-// r components in steps of 8: lane (row = l%32, half = l/32) loads
-// X[row][k0 + 4*half .. +3], and MFMA step s contracts the component pair
-// (k0 + s, k0 + 4 + s) against the matching two rows of G.
+// A workgroup stages a column chunk of G (all r rows, 32*NB columns) in LDS once
+// and then walks over 128-row tiles of X; each of its 4 waves owns 32 rows and
+// NB MFMA blocks (32*NB output columns).  The contraction runs over the r
+// components in steps of 8: lane (row = l%32, half = l/32) loads
+// X[row][k0 + 4*half .. +3] straight from global memory, and MFMA step s
+// contracts the component pair (k0 + s, k0 + 4 + s) against the matching two
+// rows of G.  In LDS the chunk is stored as [k][l%32][block], so one ds_read of
+// NB floats gives a lane its B operands of all NB blocks for one step.  The
+// multiplicative update is applied in the epilogue, so X G is never written.
 // ---------------------------------------------------------------------------
-template <bool VEC4>
-__global__ void __launch_bounds__(256)
+template <int NB>
+struct GVec;
+template <>
+struct GVec<4> { typedef float4 type; };
+template <>
+struct GVec<2> { typedef float2 type; };
+template <>
+struct GVec<1> { typedef float type; };
+
+template <int NB>
+__device__ inline void load_g(const float* p, float (&g)[NB]) {
+  typename GVec<NB>::type v = *reinterpret_cast<const typename GVec<NB>::type*>(p);
+  if constexpr (NB == 4) { g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w; }
+  else if constexpr (NB == 2) { g[0] = v.x; g[1] = v.y; }
+  else { g[0] = v; }
+}
+
+template <int NB, int PD, bool VEC4>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_xg_mu(const float* __restrict__ X, const float* __restrict__ G, const float* num, float eps,
-            int64_t rows, int r, float* out,
-            float* __restrict__ D_out) {
+            int64_t rows, int r, int nsteps, float* out, float* __restrict__ D_out) {
+  extern __shared__ float g_lds[];  // [8 * nsteps][32][NB]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
-  const int64_t row0 = (int64_t)blockIdx.x * 128 + wave * 32;
-  if (row0 >= rows) return;
-  const int c0 = blockIdx.y * 128;
-  const int64_t arow = row0 + l32;
-  const bool arow_ok = arow < rows;
-  const float* xrow = X + (arow_ok ? arow : 0) * (int64_t)r;
+  constexpr int CW = 32 * NB;
+  const int c0 = blockIdx.y * CW;
+  const int kpad = 8 * nsteps;
 
-  acc16 acc[4];
-  for (int i = 0; i < 4; i++)
-    for (int v = 0; v < 16; v++) acc[i][v] = 0.0f;
+  for (int idx = threadIdx.x; idx < kpad * CW; idx += 256) {
+    const int k = idx / CW, c = idx % CW, gc = c0 + c;
+    const float v = (k < r && gc < r) ? G[(int64_t)k * r + gc] : 0.0f;
+    g_lds[(k * 32 + (c & 31)) * NB + (c >> 5)] = v;
+  }
+  __syncthreads();
 
-  bool cok[4];
-  for (int i = 0; i < 4; i++) cok[i] = (c0 + 32 * i + l32) < r;
+  bool cok[NB];
+#pragma unroll
+  for (int i = 0; i < NB; i++) cok[i] = (c0 + 32 * i + l32) < r;
 
-  for (int k0 = 0; k0 < r; k0 += 8) {
-    const int kk = k0 + 4 * half;
-    float xa[4];
+  const int64_t n_tiles = (rows + 127) / 128;
+
+  // A operands of step `step` of tile `tile`: X[row][8 step + 4 half .. +3] (zeros outside X).
+  auto load_x = [&](int64_t tile, int step, float (&xa)[4]) {
+    const int64_t arow = tile * 128 + wave * 32 + l32;
+    const bool ok = tile < n_tiles && arow < rows;
+    const float* xrow = X + (ok ? arow : 0) * (int64_t)r;
+    const int kk = 8 * step + 4 * half;
     if (VEC4) {
-      // r % 8 == 0 here, so kk + 3 < r
-      float4 t = arow_ok ? *reinterpret_cast<const float4*>(xrow + kk) : make_float4(0, 0, 0, 0);
+      // r % 8 == 0 here, so kk + 3 < r whenever 8 step < r
+      float4 t = (ok && 8 * step < r) ? *reinterpret_cast<const float4*>(xrow + kk)
+                                      : make_float4(0, 0, 0, 0);
       xa[0] = t.x; xa[1] = t.y; xa[2] = t.z; xa[3] = t.w;
     } else {
 #pragma unroll
-      for (int s = 0; s < 4; s++) xa[s] = (arow_ok && kk + s < r) ? xrow[kk + s] : 0.0f;
+      for (int s = 0; s < 4; s++) xa[s] = (ok && kk + s < r) ? xrow[kk + s] : 0.0f;
     }
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const int kg = kk + s;
-      const bool kok = kg < r;
-      const float* grow = G + (int64_t)(kok ? kg : 0) * r + c0 + l32;
-      float g0 = (kok && cok[0]) ? grow[0] : 0.0f;
-      float g1 = (kok && cok[1]) ? grow[32] : 0.0f;
-      float g2 = (kok && cok[2]) ? grow[64] : 0.0f;
-      float g3 = (kok && cok[3]) ? grow[96] : 0.0f;
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[s], g0, acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[s], g1, acc[1], 0, 0, 0);
-      acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[s], g2, acc[2], 0, 0, 0);
-      acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[s], g3, acc[3], 0, 0, 0);
-    }
-  }
+  };
 
-  for (int i = 0; i < 4; i++) {
-    if (!cok[i]) continue;
-    const int col = c0 + 32 * i + l32;
-    for (int v = 0; v < 16; v++) {
-      int64_t row = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
-      if (row < rows) {
-        int64_t idx = row * (int64_t)r + col;
-        float d = acc[i][v];
-        float x = X[idx];
-        float q = num[idx] / (d + eps);
-        out[idx] = x * q;
-        if (D_out) D_out[idx] = d;
+  // The X operands form one stream over (tile, step); PD steps are kept in flight, across the
+  // epilogue and into the next tile, so the MFMAs never wait for a fresh global load.
+  float xq[PD][4];
+  int64_t tile = blockIdx.x;
+#pragma unroll
+  for (int d = 0; d < PD; d++) load_x(tile, d, xq[d]);
+
+  while (tile < n_tiles) {
+    const int64_t next_tile = tile + gridDim.x;
+    const int64_t row0 = tile * 128 + wave * 32;
+    acc16 acc[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+      for (int v = 0; v < 16; v++) acc[i][v] = 0.0f;
+
+    // Epilogue operands (numerator and X in the accumulator layout) are requested now and
+    // arrive while the MFMAs run.
+    float pn[NB][16], px[NB][16];
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+      const int col = c0 + 32 * i + l32;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int64_t row = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        const bool ok = cok[i] && row < rows;
+        const int64_t idx = ok ? row * (int64_t)r + col : 0;
+        pn[i][v] = ok ? num[idx] : 0.0f;
+        px[i][v] = ok ? X[idx] : 0.0f;
       }
     }
+
+    for (int s0 = 0; s0 < nsteps; s0 += PD) {
+      const bool last_round = s0 + PD >= nsteps;
+#pragma unroll
+      for (int d = 0; d < PD; d++) {
+        const int step = s0 + d;
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          float g[NB];
+          load_g<NB>(g_lds + ((8 * step + 4 * half + s) * 32 + l32) * NB, g);
+#pragma unroll
+          for (int i = 0; i < NB; i++)
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(xq[d][s], g[i], acc[i], 0, 0, 0);
+        }
+        if (last_round)
+          load_x(next_tile, d, xq[d]);
+        else
+          load_x(tile, step + PD, xq[d]);
+      }
+    }
+
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+      if (!cok[i]) continue;
+      const int col = c0 + 32 * i + l32;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int64_t row = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        if (row < rows) {
+          const int64_t idx = row * (int64_t)r + col;
+          const float d = acc[i][v];
+          const float q = pn[i][v] / (d + eps);
+          out[idx] = px[i][v] * q;
+          if (D_out) D_out[idx] = d;
+        }
+      }
+    }
+    tile = next_tile;
   }
+}
+
+template <int NB, int PD, bool VEC4>
+static int launch_xg_mu_inst(dim3 grid, size_t lds, const float* X, const float* G,
+                             const float* num, float eps, int64_t rows, int r, int nsteps,
+                             float* out, float* D_out) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu<NB, PD, VEC4>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((k_xg_mu<NB, PD, VEC4>), grid, dim3(256), lds, stream(), X, G, num, eps, rows,
+                     r, nsteps, out, D_out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int NB>
+static int launch_xg_mu_nb(int64_t rows, int r, const float* X, const float* G, const float* num,
+                           float eps, float* out, float* D_out) {
+  int nsteps = (r + 7) / 8;
+  if (nsteps > 2 && (nsteps & 1)) nsteps++;  // zero-padded, so that two steps can be in flight
+  const int pd = nsteps % 4 == 0 ? 4 : nsteps % 2 == 0 ? 2 : 1;
+  const size_t lds = (size_t)nsteps * 8 * 32 * NB * sizeof(float);
+  const bool vec4 = (r % 8 == 0) && ((uintptr_t)X % 16 == 0);
+  int64_t tiles = ceil_div(rows, 128);
+  int64_t wgs = (int64_t)n_cus() * (lds <= 72 * 1024 ? 2 : 1);
+  if (wgs > tiles) wgs = tiles;
+  dim3 grid((unsigned)wgs, (unsigned)ceil_div(r, 32 * NB));
+#define DN_XG(PDV)                                                                              \
+  (vec4 ? launch_xg_mu_inst<NB, PDV, true>(grid, lds, X, G, num, eps, rows, r, nsteps, out, D_out) \
+        : launch_xg_mu_inst<NB, PDV, false>(grid, lds, X, G, num, eps, rows, r, nsteps, out, D_out))
+  switch (pd) {
+    case 4: return DN_XG(4);
+    case 2: return DN_XG(2);
+    default: return DN_XG(1);
+  }
+#undef DN_XG
 }
 
 int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const float* num, float eps,
                  float* out, float* D_out) {
-  DN_CHECK(r >= 1 && r <= 4096, "rank %d outside [1, 4096]", r);
+  DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
   DN_CHECK(out != X, "xg_mu: out must not alias X");
   if (rows <= 0) return 0;
-  dim3 grid((unsigned)ceil_div(rows, 128), (unsigned)ceil_div(r, 128));
-  if (r % 8 == 0 && ((uintptr_t)X % 16 == 0))
-    hipLaunchKernelGGL((k_xg_mu<true>), grid, dim3(256), 0, stream(), X, G, num, eps, rows, r, out,
-                       D_out);
-  else
-    hipLaunchKernelGGL((k_xg_mu<false>), grid, dim3(256), 0, stream(), X, G, num, eps, rows, r,
-                       out, D_out);
-  DN_LAUNCH_CHECK();
-  return 0;
+  // widest column chunk whose slice of G fits 128 KB of LDS
+  if (r <= 256) return launch_xg_mu_nb<4>(rows, r, X, G, num, eps, out, D_out);
+  if (r <= 512) return launch_xg_mu_nb<2>(rows, r, X, G, num, eps, out, D_out);
+  return launch_xg_mu_nb<1>(rows, r, X, G, num, eps, out, D_out);
 }
 
 // ---------------------------------------------------------------------------
@@ -367,6 +469,22 @@ DN_API float dnpeff_uniform_at(uint64_t seed, int matrix_id, int64_t row, int64_
 DN_API int dnpeff_op_mu(int64_t count, float* F, const float* num, const float* den, float eps) {
   clear_error();
   return launch_mu(count, F, num, den, eps);
+}
+
+__global__ void __launch_bounds__(256)
+    k_copy(int64_t count, const float* __restrict__ src, float* __restrict__ dst) {
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += stride) dst[i] = src[i];
+}
+
+DN_API int dnpeff_op_copy(int64_t count, const float* src, float* dst) {
+  clear_error();
+  if (count <= 0) return 0;
+  int64_t g = ceil_div(count, 256);
+  if (g > 65536 * 16) g = 65536 * 16;
+  hipLaunchKernelGGL(k_copy, dim3((unsigned)g), dim3(256), 0, stream(), count, src, dst);
+  DN_LAUNCH_CHECK();
+  return 0;
 }
 
 DN_API int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr) {
