@@ -1,10 +1,13 @@
 // Sparse kernels: A H^T (row-major CSR, gather rows of H), A^T W (transposed
 // CSR, gather rows of W, no atomics) and sparse x sparse -> dense for the
-// fixed-H learner.  A wavefront owns one output row; lane l holds components
-// l, l+64, l+128, ... so every gathered row is read as contiguous 256-byte
-// segments.  (col, val) pairs are streamed 64 at a time, one per lane, and
-// broadcast from registers.  All summation orders are fixed by the matrix
-// structure, so results are reproducible run to run.
+// fixed-H learner.  A wavefront owns one output row.  (index, value) pairs are
+// streamed 64 at a time, one per lane, and handed out from registers.  When
+// the rank is a multiple of 4 a gathered row is read as 16-byte pieces: r/4
+// lanes cover one row, so a wave fetches 64/(r/4) rows with one instruction
+// (two for r = 128) and keeps several such instructions in flight.  Other
+// ranks use 4-byte loads, lane l holding components l, l+64, ...  All
+// summation orders are fixed by the matrix structure, so results are
+// reproducible run to run.
 #include "dnpeff_internal.hpp"
 
 namespace dn {
@@ -14,54 +17,154 @@ __device__ inline float bcast_f(float v, int src_lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 
-// acc[t] += sum_{p in [p0, p1)} val[p] * X[idx[p] * r + lane + 64 t], p ascending.
+// ---------------------------------------------------------------------------
+// Gatherers: acc += sum_{p in [p0, p1)} val[p] * X[idx[p], :], then store(dst).
+// ---------------------------------------------------------------------------
+
+// Any rank: lane l holds components l + 64 t; every entry is applied by the whole wave.
 template <int VPL>
-__device__ inline void gather_rows(const int32_t* __restrict__ idx, const float* __restrict__ val,
-                                   int64_t p0, int64_t p1, const float* __restrict__ X, int r,
-                                   int lane, const bool (&ok)[VPL], float (&acc)[VPL]) {
-  for (int64_t p = p0; p < p1; p += 64) {
-    const int cnt = (p1 - p) < 64 ? (int)(p1 - p) : 64;
-    int my_i = 0;
-    float my_v = 0.0f;
-    if (lane < cnt) {
-      my_i = idx[p + lane];
-      my_v = val[p + lane];
+struct GatherDword {
+  static constexpr int UNR = VPL <= 2 ? 8 : VPL <= 4 ? 4 : 2;
+  float acc[VPL];
+  bool ok[VPL];
+  int lane;
+
+  __device__ inline void init(int lane_, int r) {
+    lane = lane_;
+#pragma unroll
+    for (int t = 0; t < VPL; t++) {
+      ok[t] = lane + 64 * t < r;
+      acc[t] = 0.0f;
     }
-    int u = 0;
-    for (; u + 4 <= cnt; u += 4) {
-      const float* x0 = X + (int64_t)bcast_i(my_i, u) * r + lane;
-      const float* x1 = X + (int64_t)bcast_i(my_i, u + 1) * r + lane;
-      const float* x2 = X + (int64_t)bcast_i(my_i, u + 2) * r + lane;
-      const float* x3 = X + (int64_t)bcast_i(my_i, u + 3) * r + lane;
-      const float a0 = bcast_f(my_v, u), a1 = bcast_f(my_v, u + 1);
-      const float a2 = bcast_f(my_v, u + 2), a3 = bcast_f(my_v, u + 3);
-      float h0[VPL], h1[VPL], h2[VPL], h3[VPL];
-#pragma unroll
-      for (int t = 0; t < VPL; t++) {
-        h0[t] = ok[t] ? x0[64 * t] : 0.0f;
-        h1[t] = ok[t] ? x1[64 * t] : 0.0f;
-        h2[t] = ok[t] ? x2[64 * t] : 0.0f;
-        h3[t] = ok[t] ? x3[64 * t] : 0.0f;
+  }
+
+  __device__ inline void run(const int32_t* __restrict__ idx, const float* __restrict__ val,
+                             int64_t p0, int64_t p1, const float* __restrict__ X, int r) {
+    for (int64_t p = p0; p < p1; p += 64) {
+      const int cnt = (p1 - p) < 64 ? (int)(p1 - p) : 64;
+      int my_i = 0;
+      float my_v = 0.0f;
+      if (lane < cnt) {
+        my_i = idx[p + lane];
+        my_v = val[p + lane];
       }
+      int u = 0;
+      for (; u + UNR <= cnt; u += UNR) {
+        float h[UNR][VPL];
+        float a[UNR];
 #pragma unroll
-      for (int t = 0; t < VPL; t++) {
-        acc[t] = fmaf(a0, h0[t], acc[t]);
-        acc[t] = fmaf(a1, h1[t], acc[t]);
-        acc[t] = fmaf(a2, h2[t], acc[t]);
-        acc[t] = fmaf(a3, h3[t], acc[t]);
+        for (int q = 0; q < UNR; q++) {
+          const float* x = X + (int64_t)bcast_i(my_i, u + q) * r + lane;
+          a[q] = bcast_f(my_v, u + q);
+#pragma unroll
+          for (int t = 0; t < VPL; t++) h[q][t] = ok[t] ? x[64 * t] : 0.0f;
+        }
+#pragma unroll
+        for (int q = 0; q < UNR; q++)
+#pragma unroll
+          for (int t = 0; t < VPL; t++) acc[t] = fmaf(a[q], h[q][t], acc[t]);
       }
-    }
-    for (; u < cnt; u++) {
-      const float* x0 = X + (int64_t)bcast_i(my_i, u) * r + lane;
-      const float a0 = bcast_f(my_v, u);
+      for (; u < cnt; u++) {
+        const float* x0 = X + (int64_t)bcast_i(my_i, u) * r + lane;
+        const float a0 = bcast_f(my_v, u);
 #pragma unroll
-      for (int t = 0; t < VPL; t++) {
-        float h = ok[t] ? x0[64 * t] : 0.0f;
-        acc[t] = fmaf(a0, h, acc[t]);
+        for (int t = 0; t < VPL; t++) {
+          float h = ok[t] ? x0[64 * t] : 0.0f;
+          acc[t] = fmaf(a0, h, acc[t]);
+        }
       }
     }
   }
-}
+
+  __device__ inline void store(float* dst) const {
+#pragma unroll
+    for (int t = 0; t < VPL; t++)
+      if (ok[t]) dst[lane + 64 * t] = acc[t];
+  }
+};
+
+// Rank a multiple of 4.  LPR lanes cover one gathered row with 16-byte loads (T
+// loads per lane when the row is wider than 64 such pieces); the wave's 64/LPR
+// lane groups take the entries of a batch round-robin, so group g applies
+// entries g, g + G, g + 2G, ... in order, and the groups are added at the end in
+// a fixed butterfly order.
+template <int LPR, int T>
+struct GatherVec4 {
+  static constexpr int G = 64 / LPR;
+  static constexpr int UNR = T >= 4 ? 1 : T == 2 ? 2 : 4;
+  float4 acc[T];
+  bool ok[T];
+  int lane, sub, grp;
+
+  __device__ inline void init(int lane_, int r) {
+    lane = lane_;
+    sub = lane % LPR;
+    grp = lane / LPR;
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+      ok[t] = 4 * (sub + 64 * t) < r;
+      acc[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  }
+
+  __device__ inline void run(const int32_t* __restrict__ idx, const float* __restrict__ val,
+                             int64_t p0, int64_t p1, const float* __restrict__ X, int r) {
+    for (int64_t p = p0; p < p1; p += 64) {
+      const int cnt = (p1 - p) < 64 ? (int)(p1 - p) : 64;
+      int my_i = 0;
+      float my_v = 0.0f;
+      if (lane < cnt) {
+        my_i = idx[p + lane];
+        my_v = val[p + lane];
+      }
+      const int nsteps = (cnt + G - 1) / G;
+      for (int q = 0; q < nsteps; q += UNR) {
+        float4 h[UNR][T];
+        float a[UNR];
+#pragma unroll
+        for (int uu = 0; uu < UNR; uu++) {
+          const int u = (q + uu) * G + grp;
+          const bool valid = u < cnt;
+          const int j = __shfl(my_i, u & 63);
+          a[uu] = __shfl(my_v, u & 63);
+          const float* x = X + (int64_t)j * r + 4 * sub;
+#pragma unroll
+          for (int t = 0; t < T; t++)
+            h[uu][t] = (valid && ok[t]) ? *reinterpret_cast<const float4*>(x + 256 * t)
+                                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          if (!valid) a[uu] = 0.0f;
+        }
+#pragma unroll
+        for (int uu = 0; uu < UNR; uu++)
+#pragma unroll
+          for (int t = 0; t < T; t++) {
+            acc[t].x = fmaf(a[uu], h[uu][t].x, acc[t].x);
+            acc[t].y = fmaf(a[uu], h[uu][t].y, acc[t].y);
+            acc[t].z = fmaf(a[uu], h[uu][t].z, acc[t].z);
+            acc[t].w = fmaf(a[uu], h[uu][t].w, acc[t].w);
+          }
+      }
+    }
+  }
+
+  __device__ inline void store(float* dst) {
+#pragma unroll
+    for (int off = 32; off >= LPR; off >>= 1) {
+#pragma unroll
+      for (int t = 0; t < T; t++) {
+        acc[t].x += __shfl_xor(acc[t].x, off);
+        acc[t].y += __shfl_xor(acc[t].y, off);
+        acc[t].z += __shfl_xor(acc[t].z, off);
+        acc[t].w += __shfl_xor(acc[t].w, off);
+      }
+    }
+    if (grp == 0) {
+#pragma unroll
+      for (int t = 0; t < T; t++)
+        if (ok[t]) *reinterpret_cast<float4*>(dst + 4 * (sub + 64 * t)) = acc[t];
+    }
+  }
+};
 
 // Row that owns work chunk `chunk`: chunk_base[row] <= chunk < chunk_base[row + 1].
 __device__ inline int64_t chunk_to_row(const int64_t* __restrict__ chunk_base, int64_t n_rows,
@@ -74,17 +177,19 @@ __device__ inline int64_t chunk_to_row(const int64_t* __restrict__ chunk_base, i
   return lo;
 }
 
+constexpr int MAX_RANK = 1024;
+
 // ---------------------------------------------------------------------------
 // partials[chunk, :] = sum over the chunk's entries of val * H[col, :]
 // A workgroup owns SPMM_N_CHUNK consecutive entries of one row; its 4 waves
 // take a quarter each and are combined in wave order.
 // ---------------------------------------------------------------------------
-template <int VPL>
+template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_n(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
              const float* __restrict__ vals, const int64_t* __restrict__ chunk_base, int64_t n_rows,
              int r, const float* __restrict__ H, float* __restrict__ partials) {
-  __shared__ float red[4][64 * VPL];
+  extern __shared__ __align__(16) float red_dyn[];  // [4][r]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int64_t chunk = blockIdx.x;
   const int64_t row = chunk_to_row(chunk_base, n_rows, chunk);
@@ -96,22 +201,16 @@ __global__ void __launch_bounds__(256)
   if (w0 > e1) w0 = e1;
   if (w1 > e1) w1 = e1;
 
-  bool ok[VPL];
-  float acc[VPL];
-#pragma unroll
-  for (int t = 0; t < VPL; t++) {
-    ok[t] = lane + 64 * t < r;
-    acc[t] = 0.0f;
-  }
-  gather_rows<VPL>(colind, vals, w0, w1, H, r, lane, ok, acc);
-#pragma unroll
-  for (int t = 0; t < VPL; t++) red[wave][lane + 64 * t] = acc[t];
+  GT g;
+  g.init(lane, r);
+  g.run(colind, vals, w0, w1, H, r);
+  g.store(red_dyn + wave * r);
   __syncthreads();
   for (int c = threadIdx.x; c < r; c += 256) {
-    float s = red[0][c];
-    s += red[1][c];
-    s += red[2][c];
-    s += red[3][c];
+    float s = red_dyn[c];
+    s += red_dyn[r + c];
+    s += red_dyn[2 * r + c];
+    s += red_dyn[3 * r + c];
     partials[chunk * r + c] = s;
   }
 }
@@ -132,7 +231,7 @@ __global__ void __launch_bounds__(256)
 // ---------------------------------------------------------------------------
 // T[j, :] = sum over column j's entries (ascending row) of val * W[row, :]
 // ---------------------------------------------------------------------------
-template <int VPL>
+template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_short(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
                    const float* __restrict__ tvals, int64_t m, int r, const float* __restrict__ W,
@@ -142,25 +241,18 @@ __global__ void __launch_bounds__(256)
   if (j >= m) return;
   const int64_t p0 = colptr[j], p1 = colptr[j + 1];
   if (p1 - p0 > SPMM_T_LONG) return;  // written by k_spmm_t_long
-  bool ok[VPL];
-  float acc[VPL];
-#pragma unroll
-  for (int t = 0; t < VPL; t++) {
-    ok[t] = lane + 64 * t < r;
-    acc[t] = 0.0f;
-  }
-  gather_rows<VPL>(rowind, tvals, p0, p1, W, r, lane, ok, acc);
-#pragma unroll
-  for (int t = 0; t < VPL; t++)
-    if (ok[t]) T[j * r + lane + 64 * t] = acc[t];
+  GT g;
+  g.init(lane, r);
+  g.run(rowind, tvals, p0, p1, W, r);
+  g.store(T + j * r);
 }
 
-template <int VPL>
+template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_long(const int32_t* __restrict__ long_cols, const int64_t* __restrict__ colptr,
                   const int32_t* __restrict__ rowind, const float* __restrict__ tvals, int r,
                   const float* __restrict__ W, float* __restrict__ T) {
-  __shared__ float red[4][64 * VPL];
+  extern __shared__ __align__(16) float red_dyn[];  // [4][r]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int64_t j = long_cols[blockIdx.x];
   const int64_t p0 = colptr[j], p1 = colptr[j + 1];
@@ -168,22 +260,16 @@ __global__ void __launch_bounds__(256)
   int64_t w0 = p0 + wave * per, w1 = w0 + per;
   if (w0 > p1) w0 = p1;
   if (w1 > p1) w1 = p1;
-  bool ok[VPL];
-  float acc[VPL];
-#pragma unroll
-  for (int t = 0; t < VPL; t++) {
-    ok[t] = lane + 64 * t < r;
-    acc[t] = 0.0f;
-  }
-  gather_rows<VPL>(rowind, tvals, w0, w1, W, r, lane, ok, acc);
-#pragma unroll
-  for (int t = 0; t < VPL; t++) red[wave][lane + 64 * t] = acc[t];
+  GT g;
+  g.init(lane, r);
+  g.run(rowind, tvals, w0, w1, W, r);
+  g.store(red_dyn + wave * r);
   __syncthreads();
   for (int c = threadIdx.x; c < r; c += 256) {
-    float s = red[0][c];
-    s += red[1][c];
-    s += red[2][c];
-    s += red[3][c];
+    float s = red_dyn[c];
+    s += red_dyn[r + c];
+    s += red_dyn[2 * r + c];
+    s += red_dyn[3 * r + c];
     T[j * r + c] = s;
   }
 }
@@ -295,25 +381,46 @@ static int vpl_for(int r) {
   return p;
 }
 
-#define DN_DISPATCH_VPL(vpl, CALL)                        \
-  switch (vpl) {                                          \
-    case 1: { constexpr int V = 1; CALL; } break;         \
-    case 2: { constexpr int V = 2; CALL; } break;         \
-    case 4: { constexpr int V = 4; CALL; } break;         \
-    case 8: { constexpr int V = 8; CALL; } break;         \
-    case 16: { constexpr int V = 16; CALL; } break;       \
-    default: set_error("rank too large for the sparse kernels (max 1024)"); return 2; \
+template <class T>
+struct TypeTag {
+  using type = T;
+};
+
+// Calls f(TypeTag<Gatherer>) with the gatherer that fits rank r and the alignment of X.
+template <class F>
+static int dispatch_gather(int r, bool aligned16, F&& f) {
+  if (r % 4 == 0 && aligned16) {
+    const int r4 = r / 4;
+    if (r4 <= 4) return f(TypeTag<GatherVec4<4, 1>>{});
+    if (r4 <= 8) return f(TypeTag<GatherVec4<8, 1>>{});
+    if (r4 <= 16) return f(TypeTag<GatherVec4<16, 1>>{});
+    if (r4 <= 32) return f(TypeTag<GatherVec4<32, 1>>{});
+    if (r4 <= 64) return f(TypeTag<GatherVec4<64, 1>>{});
+    if (r4 <= 128) return f(TypeTag<GatherVec4<64, 2>>{});
+    return f(TypeTag<GatherVec4<64, 4>>{});
   }
+  switch (vpl_for(r)) {
+    case 1: return f(TypeTag<GatherDword<1>>{});
+    case 2: return f(TypeTag<GatherDword<2>>{});
+    case 4: return f(TypeTag<GatherDword<4>>{});
+    case 8: return f(TypeTag<GatherDword<8>>{});
+    default: return f(TypeTag<GatherDword<16>>{});
+  }
+}
 
 int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr, float* /*N_nr*/, float* partials) {
-  DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
+  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   DN_CHECK(A->rowptr && A->chunk_base, "matrix has no row-major copy / work list");
   if (A->n_chunks == 0) return 0;
   DN_CHECK(A->n_chunks < (int64_t)INT32_MAX, "too many work chunks");
   dim3 grid((unsigned)A->n_chunks), block(256);
-  DN_DISPATCH_VPL(vpl_for(r), hipLaunchKernelGGL((k_spmm_n<V>), grid, block, 0, stream(), A->rowptr,
-                                                 A->colind, A->vals, A->chunk_base, A->n_rows, r,
-                                                 H_mr, partials));
+  const size_t lds = sizeof(float) * 4 * (size_t)r;
+  dispatch_gather(r, ((uintptr_t)H_mr % 16) == 0, [&](auto tag) {
+    using GT = typename decltype(tag)::type;
+    hipLaunchKernelGGL((k_spmm_n<GT>), grid, block, lds, stream(), A->rowptr, A->colind, A->vals,
+                       A->chunk_base, A->n_rows, r, H_mr, partials);
+    return 0;
+  });
   DN_LAUNCH_CHECK();
   return 0;
 }
@@ -327,35 +434,47 @@ int launch_spmm_n_reduce(const dnpeff_csr* A, int r, const float* partials, floa
 }
 
 int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
-  DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
+  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   DN_CHECK(A->colptr != nullptr, "matrix has no transposed copy");
   if (A->n_cols == 0) return 0;
   dim3 grid((unsigned)ceil_div(A->n_cols, 4)), block(256);
-  DN_DISPATCH_VPL(vpl_for(r), hipLaunchKernelGGL((k_spmm_t_short<V>), grid, block, 0, stream(),
-                                                 A->colptr, A->rowind, A->tvals, A->n_cols, r,
-                                                 W_nr, T_mr));
-  if (A->n_long > 0) {
-    dim3 grid_l((unsigned)A->n_long);
-    DN_DISPATCH_VPL(vpl_for(r), hipLaunchKernelGGL((k_spmm_t_long<V>), grid_l, block, 0, stream(),
-                                                   A->long_cols, A->colptr, A->rowind, A->tvals, r,
-                                                   W_nr, T_mr));
-  }
+  const bool aligned = ((uintptr_t)T_mr % 16) == 0 && ((uintptr_t)W_nr % 16) == 0;
+  dispatch_gather(r, aligned, [&](auto tag) {
+    using GT = typename decltype(tag)::type;
+    hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), A->colptr, A->rowind,
+                       A->tvals, A->n_cols, r, W_nr, T_mr);
+    if (A->n_long > 0) {
+      dim3 grid_l((unsigned)A->n_long);
+      const size_t lds = sizeof(float) * 4 * (size_t)r;
+      hipLaunchKernelGGL((k_spmm_t_long<GT>), grid_l, block, lds, stream(), A->long_cols,
+                         A->colptr, A->rowind, A->tvals, r, W_nr, T_mr);
+    }
+    return 0;
+  });
   DN_LAUNCH_CHECK();
   return 0;
 }
 
 int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials) {
   const int r = (int)B->n_rows;
-  DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
+  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   DN_CHECK(A->rowptr && A->chunk_base, "matrix has no row-major copy / work list");
   DN_CHECK(B->colptr != nullptr, "sparse factor has no transposed copy");
   DN_CHECK(A->n_cols == B->n_cols, "column counts differ (%lld vs %lld)", (long long)A->n_cols,
            (long long)B->n_cols);
   if (A->n_chunks == 0) return 0;
   dim3 grid((unsigned)A->n_chunks), block(256);
-  DN_DISPATCH_VPL(vpl_for(r), hipLaunchKernelGGL((k_spsp<V>), grid, block, 0, stream(), A->rowptr,
-                                                 A->colind, A->vals, A->chunk_base, A->n_rows, r,
-                                                 B->colptr, B->rowind, B->tvals, partials));
+#define DN_SPSP(V)                                                                              \
+  hipLaunchKernelGGL((k_spsp<V>), grid, block, 0, stream(), A->rowptr, A->colind, A->vals,        \
+                     A->chunk_base, A->n_rows, r, B->colptr, B->rowind, B->tvals, partials)
+  switch (vpl_for(r)) {
+    case 1: DN_SPSP(1); break;
+    case 2: DN_SPSP(2); break;
+    case 4: DN_SPSP(4); break;
+    case 8: DN_SPSP(8); break;
+    default: DN_SPSP(16); break;
+  }
+#undef DN_SPSP
   DN_LAUNCH_CHECK();
   return 0;
 }
