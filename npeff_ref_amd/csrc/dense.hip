@@ -5,6 +5,8 @@
 #include "dnpeff_internal.hpp"
 #include "synth_rng.h"
 
+#include <type_traits>
+
 namespace dn {
 
 typedef float acc16 __attribute__((ext_vector_type(16)));
@@ -32,17 +34,22 @@ int launch_mu(int64_t count, float* F, const float* num, const float* den, float
 // ---------------------------------------------------------------------------
 // Gram  G = X^T X
 //
-// One workgroup (4 waves) owns a 128 x 128 tile of G over a slice of the rows of
-// X; wave w owns the 64 x 64 quadrant (w/2, w%2) as 2 x 2 MFMA blocks.  Operand
-// layout of v_mfma_f32_32x32x2f32: lane l supplies A[i = l%32][k = l/32] and
-// B[k = l/32][j = l%32]; both come straight from two consecutive rows of X, so
-// every load is a pair of 128-byte row segments.  Accumulators are flushed into
-// a second set every GRAM_FLUSH rows so no fp32 running sum grows long.  Slice
-// partials are summed in fp64 in slice order by k_gram_reduce.
+// v_mfma_f32_32x32x2f32 takes from lane l the element A[i = l%32][k = l/32] and
+// B[k = l/32][j = l%32].  Here k runs over two consecutive rows of X and the 32
+// "columns" of an operand block are every fourth column of a 128-column tile:
+// strided block sb = 4 t + a holds columns 128 t + 4 i + a, i < 32.  Lane l then
+// needs X[k + l/32][128 t + 4 (l%32) + a] for a = 0..3: ONE 16-byte load per lane
+// and row pair feeds all four strided blocks of the tile, i.e. the A and B
+// operands of up to 16 MFMAs, and 16-byte loads are the only form that reaches
+// the L1's full rate.  G is symmetric, so only block pairs (sbi <= sbj) are
+// computed; the reduce kernel mirrors and un-strides them.  Pairs are numbered
+// row by row; a wave owns two consecutive pairs over a slice of the rows of X, a
+// workgroup of 5 waves owns 10 (all of G for r <= 128).  Accumulators are flushed
+// are kept per slice (at most rows / 2048 rows each), and the slice partials are summed in
+// fp64 in slice order by k_gram_reduce, so no fp32 running sum grows long.
 // ---------------------------------------------------------------------------
-constexpr int GRAM_TILE = 128;
-constexpr int64_t GRAM_FLUSH = 4096;
-constexpr int GRAM_MAX_SLICES = 1024;
+constexpr int GRAM_MAX_SLICES = 2048;
+constexpr int GRAM_UNR = 8;  // row pairs in flight per wave
 
 static int64_t gram_slices(int64_t rows) {
   int64_t s = ceil_div(rows, 256);
@@ -51,112 +58,324 @@ static int64_t gram_slices(int64_t rows) {
   return s;
 }
 
+__host__ __device__ inline int gram_blocks(int r) { return 4 * ((r + 127) / 128); }
+// Number of the block pair (bi <= bj) in row-major order over the upper triangle.
+__host__ __device__ inline int gram_pair_index(int bi, int bj, int nb) {
+  return bi * nb - bi * (bi - 1) / 2 + (bj - bi);
+}
+static int gram_pairs(int r) {
+  int nb = gram_blocks(r);
+  return nb * (nb + 1) / 2;
+}
+
 int64_t gram_workspace_floats(int64_t rows, int r) {
-  int64_t tiles = ceil_div(r, GRAM_TILE);
-  return gram_slices(rows) * tiles * tiles * GRAM_TILE * GRAM_TILE;
+  return gram_slices(rows) * (int64_t)gram_pairs(r) * 1024;
 }
 
-__global__ void __launch_bounds__(256)
-    k_gram(const float* __restrict__ X, int64_t rows, int r, int64_t rows_per_slice, int tiles,
-           float* __restrict__ partials) {
-  const int slice = blockIdx.x;
-  const int tile_a = blockIdx.y / tiles, tile_b = blockIdx.y % tiles;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+template <int A>
+__device__ inline float comp4(const float4& v) {
+  return A == 0 ? v.x : A == 1 ? v.y : A == 2 ? v.z : v.w;
+}
+
+constexpr int GRAM_TILE_FLOATS = 4096;  // one LDS slot: KB rows x ld columns (16 KB)
+constexpr int GRAM_STAGES = 3;          // row tiles in flight in registers
+constexpr int GRAM_NP = 3;              // block pairs per wave
+
+// LDS position of column c of a row: the four strided blocks of a 128-column tile are stored
+// one after the other, 32 floats each, so that the 32 lanes reading one block touch 32
+// different banks.
+__device__ inline int gram_lds_col(int c) { return (c & ~127) + 32 * (c & 3) + ((c & 127) >> 2); }
+
+// Streams row tiles of X through two LDS slots of `kb` rows each.  Every element is read from
+// global memory once per workgroup, with 16-byte loads issued GRAM_STAGES tiles ahead of their
+// use (global latency is several microseconds, one tile of MFMAs lasts about one), parked in
+// registers and written to the free LDS slot one tile ahead.
+template <int NW, bool VEC4>
+struct GramPipe {
+  static constexpr int THREADS = 64 * NW;
+  static constexpr int NVEC = (GRAM_TILE_FLOATS / 4 + THREADS - 1) / THREADS;
+  const float* __restrict__ X;
+  int r, ld, kb;
+  int64_t k1;  // number of rows of X
+  float4 stage[GRAM_STAGES][NVEC];
+
+  __device__ inline void fetch(int st, int64_t kt) {
+    if (!VEC4) return;
+    const int r4 = r >> 2;
+#pragma unroll
+    for (int q = 0; q < NVEC; q++) {
+      const int f = threadIdx.x + q * THREADS;
+      const int64_t row = kt + f / r4;
+      const bool ok = f < kb * r4 && row < k1;
+      stage[st][q] = ok ? *reinterpret_cast<const float4*>(X + row * (int64_t)r + 4 * (f % r4))
+                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  }
+  __device__ inline void commit(int st, float* slot, int64_t kt) {
+    if (VEC4) {
+      const int r4 = r >> 2;
+#pragma unroll
+      for (int q = 0; q < NVEC; q++) {
+        const int f = threadIdx.x + q * THREADS;
+        if (f < kb * r4) {
+          const int c4 = f % r4;  // columns 4 c4 .. 4 c4 + 3 = position c4 % 32 of blocks 0..3
+          float* p = slot + (f / r4) * ld + (c4 >> 5) * 128 + (c4 & 31);
+          p[0] = stage[st][q].x;
+          p[32] = stage[st][q].y;
+          p[64] = stage[st][q].z;
+          p[96] = stage[st][q].w;
+        }
+      }
+    } else {
+      for (int e = threadIdx.x; e < kb * r; e += THREADS) {
+        const int64_t row = kt + e / r;
+        const int c = e % r;
+        slot[(e / r) * ld + gram_lds_col(c)] = row < k1 ? X[row * (int64_t)r + c] : 0.0f;
+      }
+    }
+  }
+};
+
+struct GramPairs {  // strided-block residues of a wave's block pairs within its tile pair
+  int a[GRAM_NP], b[GRAM_NP], n;
+};
+
+// MFMAs of one LDS slot for the wave's NP block pairs.  KB > 0, LD > 0: tile height and LDS row
+// length known at compile time (the loop is fully unrolled, LDS reads carry immediate offsets
+// and are scheduled ahead of the MFMAs of the previous row group); KB = 0: run-time values.
+template <int NP, int KB, int LD>
+__device__ inline void gram_tile_mfma(const float* __restrict__ slot, int kb_rt, int ld_rt, int ta,
+                                      int tb, const GramPairs& gp, int lane, acc16 (&acc)[GRAM_NP]) {
   const int l32 = lane & 31, half = lane >> 5;
-  const int ca = tile_a * GRAM_TILE + (wave >> 1) * 64 + l32;  // column of X feeding A, block 0
-  const int cb = tile_b * GRAM_TILE + (wave & 1) * 64 + l32;   // column of X feeding B, block 0
-  const bool a0ok = ca < r, a1ok = ca + 32 < r, b0ok = cb < r, b1ok = cb + 32 < r;
-
-  int64_t k0 = (int64_t)slice * rows_per_slice;
-  int64_t k1 = k0 + rows_per_slice;
-  if (k1 > rows) k1 = rows;
-
-  acc16 acc[4], tot[4];
-  for (int i = 0; i < 4; i++)
-    for (int v = 0; v < 16; v++) {
-      acc[i][v] = 0.0f;
-      tot[i][v] = 0.0f;
-    }
-
-  for (int64_t kf = k0; kf < k1; kf += GRAM_FLUSH) {
-    int64_t kend = kf + GRAM_FLUSH < k1 ? kf + GRAM_FLUSH : k1;
-    int64_t k = kf;
-    // full groups of 8 row pairs, loads issued ahead of the MFMAs
-    for (; k + 16 <= kend; k += 16) {
-      float a0[8], a1[8], b0[8], b1[8];
+  const int ld = KB > 0 ? LD : ld_rt;
+  const int kb = KB > 0 ? KB : kb_rt;
+  const float* pa[NP];
+  const float* pb[NP];
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        const float* row = X + (k + 2 * u + half) * (int64_t)r;
-        a0[u] = a0ok ? row[ca] : 0.0f;
-        a1[u] = a1ok ? row[ca + 32] : 0.0f;
-        b0[u] = b0ok ? row[cb] : 0.0f;
-        b1[u] = b1ok ? row[cb + 32] : 0.0f;
-      }
-#pragma unroll
-      for (int u = 0; u < 8; u++) {
-        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[u], b0[u], acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[u], b1[u], acc[1], 0, 0, 0);
-        acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[u], b0[u], acc[2], 0, 0, 0);
-        acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[u], b1[u], acc[3], 0, 0, 0);
-      }
-    }
-    for (; k < kend; k += 2) {
-      int64_t kr = k + half;
-      bool rok = kr < kend;
-      const float* row = X + kr * (int64_t)r;
-      float a0 = (rok && a0ok) ? row[ca] : 0.0f;
-      float a1 = (rok && a1ok) ? row[ca + 32] : 0.0f;
-      float b0 = (rok && b0ok) ? row[cb] : 0.0f;
-      float b1 = (rok && b1ok) ? row[cb + 32] : 0.0f;
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[1], 0, 0, 0);
-      acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[2], 0, 0, 0);
-      acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[3], 0, 0, 0);
-    }
-    for (int i = 0; i < 4; i++)
-      for (int v = 0; v < 16; v++) {
-        tot[i][v] += acc[i][v];
-        acc[i][v] = 0.0f;
-      }
+  for (int i = 0; i < NP; i++) {
+    pa[i] = slot + half * ld + 128 * ta + 32 * gp.a[i] + l32;
+    pb[i] = slot + half * ld + 128 * tb + 32 * gp.b[i] + l32;
   }
-
-  // D layout of the 32x32 block: reg v of lane l holds row 8*(v/4) + 4*(l/32) + v%4,
-  // column l%32.
-  float* out = partials + ((int64_t)slice * tiles * tiles + blockIdx.y) * (GRAM_TILE * GRAM_TILE);
-  for (int i = 0; i < 4; i++) {
-    int rb = (wave >> 1) * 64 + (i >> 1) * 32;
-    int cbk = (wave & 1) * 64 + (i & 1) * 32;
-    for (int v = 0; v < 16; v++) {
-      int rr = rb + 8 * (v >> 2) + 4 * half + (v & 3);
-      out[rr * GRAM_TILE + cbk + l32] = tot[i][v];
+  if (KB > 0) {
+    constexpr int GRP = 4;  // row pairs whose operands are read together
+#pragma unroll
+    for (int g = 0; g < KB / 2; g += GRP) {
+      float xa[GRP][NP], xb[GRP][NP];
+#pragma unroll
+      for (int u = 0; u < GRP; u++)
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+          xa[u][i] = pa[i][2 * (g + u) * LD];
+          xb[u][i] = pb[i][2 * (g + u) * LD];
+        }
+#pragma unroll
+      for (int u = 0; u < GRP; u++)
+#pragma unroll
+        for (int i = 0; i < NP; i++)
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u][i], xb[u][i], acc[i], 0, 0, 0);
+    }
+  } else {
+    for (int kk = 0; kk < kb; kk += 2) {
+      float xa[NP], xb[NP];
+#pragma unroll
+      for (int i = 0; i < NP; i++) {
+        xa[i] = pa[i][kk * ld];
+        xb[i] = pb[i][kk * ld];
+      }
+#pragma unroll
+      for (int i = 0; i < NP; i++)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i], xb[i], acc[i], 0, 0, 0);
     }
   }
 }
 
+// The row tiles of X are dealt to the slices round-robin (slice s owns tiles s, s + S, ...), so
+// that at any moment the workgroups read one contiguous window of X.
+template <int NW, int NP, bool FAST, bool VEC4>
+__device__ inline void gram_stream(const float* __restrict__ X, int r, int kb, int64_t rows,
+                                   int slice, int n_slices, float* __restrict__ lds, int lane,
+                                   int ta, int tb, const GramPairs& gp, float* __restrict__ base,
+                                   int nb) {
+  GramPipe<NW, VEC4> pipe;
+  const int ld = 128 * ((r + 127) / 128);
+  pipe.X = X; pipe.r = r; pipe.ld = ld; pipe.kb = kb; pipe.k1 = rows;
+  const int64_t all_tiles = (rows + kb - 1) / kb;
+  const int64_t n_tiles = all_tiles > slice ? (all_tiles - slice + n_slices - 1) / n_slices : 0;
+  const int64_t k0 = (int64_t)slice * kb;         // first row of this slice's tile 0
+  const int64_t tstride = (int64_t)n_slices * kb;  // rows between consecutive tiles of the slice
+  acc16 acc[GRAM_NP];
+  for (int i = 0; i < GRAM_NP; i++)
+    for (int v = 0; v < 16; v++) acc[i][v] = 0.0f;
+  if (!VEC4 || ld != r) {  // padding columns of the LDS rows are read as operands: zero them once
+    for (int e = threadIdx.x; e < 2 * GRAM_TILE_FLOATS; e += 64 * NW) lds[e] = 0.0f;
+    __syncthreads();
+  }
+#pragma unroll
+  for (int st = 0; st < GRAM_STAGES; st++) pipe.fetch(st, k0 + (int64_t)st * tstride);
+  if (n_tiles > 0) pipe.commit(0, lds, k0);
+  __syncthreads();
+
+  // iteration t: tile t is in slot t & 1; stage[t % S] is free and receives tile t + S;
+  // tile t + 1 sits in stage[(t + 1) % S] and moves to the other slot after the MFMAs.
+  auto step = [&](int64_t t, auto st_tag) {
+    constexpr int ST = decltype(st_tag)::value;
+    pipe.fetch(ST, k0 + (t + GRAM_STAGES) * tstride);
+    gram_tile_mfma<NP, FAST ? 32 : 0, FAST ? 128 : 0>(lds + (t & 1) * GRAM_TILE_FLOATS, kb, ld, ta, tb,
+                                                       gp, lane, acc);
+    if (t + 1 < n_tiles)
+      pipe.commit((ST + 1) % GRAM_STAGES, lds + ((t + 1) & 1) * GRAM_TILE_FLOATS,
+                  k0 + (t + 1) * tstride);
+    __syncthreads();
+  };
+  int64_t t = 0;
+  for (; t + GRAM_STAGES <= n_tiles; t += GRAM_STAGES) {
+    step(t, std::integral_constant<int, 0>{});
+    step(t + 1, std::integral_constant<int, 1>{});
+    step(t + 2, std::integral_constant<int, 2>{});
+  }
+  if (t < n_tiles) step(t, std::integral_constant<int, 0>{});
+  if (t + 1 < n_tiles) step(t + 1, std::integral_constant<int, 1>{});
+
+  const int l32 = lane & 31, half = lane >> 5;
+  // D layout of the 32x32 block: reg v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+#pragma unroll
+  for (int i = 0; i < NP; i++) {
+    {
+      float* out = base + (int64_t)gram_pair_index(4 * ta + gp.a[i], 4 * tb + gp.b[i], nb) * 1024;
+      for (int v = 0; v < 16; v++) {
+        const int rr = 8 * (v >> 2) + 4 * half + (v & 3);
+        out[rr * 32 + l32] = acc[i][v];
+      }
+    }
+  }
+}
+
+// Tile pair number -> (ta <= tb), row by row over the upper triangle.
+__device__ inline void gram_tile_pair(int p, int n_tiles, int& ta, int& tb) {
+  ta = 0;
+  int row_len = n_tiles;
+  while (p >= row_len) {
+    p -= row_len;
+    ta++;
+    row_len--;
+  }
+  tb = ta + p;
+}
+
+// One workgroup of 4 waves per (tile pair, slice).  A diagonal tile pair has 10 distinct block
+// pairs (a <= b): waves take 3, 3, 3, 1.  An off-diagonal one has 16: two workgroups' worth is
+// covered by launching it twice in grid.x (sub = 0: residues a in {0, 1}, sub = 1: {2, 3}),
+// each wave taking a row half: 2 pairs.  Here: one kernel, NP chosen per wave at run time.
+template <bool VEC4>
 __global__ void __launch_bounds__(256)
-    k_gram_reduce(const float* __restrict__ partials, int64_t slices, int tiles, int r,
+    k_gram(const float* __restrict__ X, int64_t rows, int r, int kb, int n_pairs, int n_tiles,
+           float* __restrict__ partials) {
+  __shared__ __align__(16) float lds[2 * GRAM_TILE_FLOATS];
+  const int slice = blockIdx.y, n_slices = gridDim.y;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int nb = gram_blocks(r);
+  // grid.x: first the diagonal tile pairs (one workgroup each), then the off-diagonal ones
+  // (two workgroups each)
+  int ta, tb, sub = 0;
+  bool diag;
+  if ((int)blockIdx.x < n_tiles) {
+    ta = tb = blockIdx.x;
+    diag = true;
+  } else {
+    const int q = blockIdx.x - n_tiles;
+    // off-diagonal pairs (ta < tb) numbered row by row
+    int p = q >> 1, row_len = n_tiles - 1;
+    ta = 0;
+    while (p >= row_len) {
+      p -= row_len;
+      ta++;
+      row_len--;
+    }
+    tb = ta + 1 + p;
+    sub = q & 1;
+    diag = false;
+  }
+  float* base = partials + (int64_t)slice * n_pairs * 1024;
+  GramPairs gp;
+  if (diag) {
+    // (0,0)(0,1)(0,2) | (0,3)(1,1)(1,2) | (1,3)(2,2)(2,3) | (3,3)
+    const int A[4][3] = {{0, 0, 0}, {0, 1, 1}, {1, 2, 2}, {3, 3, 3}};
+    const int B[4][3] = {{0, 1, 2}, {3, 1, 2}, {3, 2, 3}, {3, 3, 3}};
+    for (int i = 0; i < 3; i++) {
+      gp.a[i] = A[wave][i];
+      gp.b[i] = B[wave][i];
+    }
+    gp.n = wave == 3 ? 1 : 3;
+  } else {
+    // residue a = 2 sub + wave / 2, b in {2 (wave % 2), 2 (wave % 2) + 1}
+    for (int i = 0; i < 3; i++) {
+      gp.a[i] = 2 * sub + (wave >> 1);
+      gp.b[i] = 2 * (wave & 1) + (i & 1);
+    }
+    gp.n = 2;
+  }
+  // r <= 128 has one tile of 128 LDS columns and 32 rows per slot: fully unrolled MFMA loop
+  if (r <= 128) {
+    if (gp.n == 3)
+      gram_stream<4, 3, true, VEC4>(X, r, kb, rows, slice, n_slices, lds, lane, ta, tb, gp, base, nb);
+    else
+      gram_stream<4, 1, true, VEC4>(X, r, kb, rows, slice, n_slices, lds, lane, ta, tb, gp, base, nb);
+  } else {
+    if (gp.n == 3)
+      gram_stream<4, 3, false, VEC4>(X, r, kb, rows, slice, n_slices, lds, lane, ta, tb, gp, base, nb);
+    else if (gp.n == 2)
+      gram_stream<4, 2, false, VEC4>(X, r, kb, rows, slice, n_slices, lds, lane, ta, tb, gp, base, nb);
+    else
+      gram_stream<4, 1, false, VEC4>(X, r, kb, rows, slice, n_slices, lds, lane, ta, tb, gp, base, nb);
+  }
+}
+
+// One thread per element of a computed block: sums its slice partials (coalesced across
+// threads) and writes the element and its mirror image.
+__global__ void __launch_bounds__(256)
+    k_gram_reduce(const float* __restrict__ partials, int64_t slices, int n_pairs, int r,
                   float* __restrict__ G) {
-  int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= r * r) return;
-  int a = idx / r, b = idx % r;
-  int tile = (a / GRAM_TILE) * tiles + (b / GRAM_TILE);
-  int off = (a % GRAM_TILE) * GRAM_TILE + (b % GRAM_TILE);
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= n_pairs * 1024) return;
+  const int nb = gram_blocks(r);
+  int pair = e >> 10, ba = 0, row_len = nb;
+  while (pair >= row_len) {
+    pair -= row_len;
+    ba++;
+    row_len--;
+  }
+  const int bb = ba + pair;
+  const int ia = (e >> 5) & 31, ib = e & 31;
+  // strided block sb holds columns 128 (sb / 4) + 4 i + sb % 4
+  const int a = 128 * (ba >> 2) + 4 * ia + (ba & 3), b = 128 * (bb >> 2) + 4 * ib + (bb & 3);
+  if (a >= r || b >= r) return;
+  const int64_t stride = (int64_t)n_pairs * 1024;
+  const float* p = partials + e;
   double s = 0.0;
-  for (int64_t sl = 0; sl < slices; sl++)
-    s += (double)partials[(sl * tiles * tiles + tile) * (GRAM_TILE * GRAM_TILE) + off];
-  G[idx] = (float)s;
+  for (int64_t sl = 0; sl < slices; sl++) s += (double)p[sl * stride];
+  G[(int64_t)a * r + b] = (float)s;
+  G[(int64_t)b * r + a] = (float)s;
 }
 
 int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace) {
   DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
-  int tiles = (int)ceil_div(r, GRAM_TILE);
+  const int n_pairs = gram_pairs(r);
+  const int n_tiles = (r + 127) / 128;
   int64_t slices = gram_slices(rows);
-  int64_t rps = ceil_div(rows > 0 ? rows : 1, slices);
-  rps = ceil_div(rps, 2) * 2;  // slices start on even rows
-  hipLaunchKernelGGL(k_gram, dim3((unsigned)slices, (unsigned)(tiles * tiles)), dim3(256), 0,
-                     stream(), X, rows, r, rps, tiles, workspace);
-  hipLaunchKernelGGL(k_gram_reduce, dim3((unsigned)ceil_div((int64_t)r * r, 256)), dim3(256), 0,
-                     stream(), workspace, slices, tiles, r, G);
+  const bool vec4 = r % 4 == 0 && ((uintptr_t)X % 16) == 0;
+  // rows per LDS slot: even, a multiple of 8 where possible, with kb * ld <= GRAM_TILE_FLOATS
+  const int ld = 128 * n_tiles;
+  int kb = GRAM_TILE_FLOATS / ld;
+  kb = kb >= 8 ? kb / 8 * 8 : kb / 2 * 2;
+  dim3 grid((unsigned)(n_tiles + n_tiles * (n_tiles - 1)), (unsigned)slices);
+  if (vec4)
+    hipLaunchKernelGGL((k_gram<true>), grid, dim3(256), 0, stream(), X, rows, r, kb, n_pairs,
+                       n_tiles, workspace);
+  else
+    hipLaunchKernelGGL((k_gram<false>), grid, dim3(256), 0, stream(), X, rows, r, kb, n_pairs,
+                       n_tiles, workspace);
+  hipLaunchKernelGGL(k_gram_reduce, dim3((unsigned)(n_pairs * 4)), dim3(256), 0, stream(), workspace,
+                     slices, n_pairs, r, G);
   DN_LAUNCH_CHECK();
   return 0;
 }
