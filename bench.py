@@ -150,7 +150,7 @@ def main():
     nmf.set_profiling(False)
     loss = nmf.computeUncachedLoss()
     ms_per_step = elapsed * 1e3 / args.steps
-    log(f"{args.steps} steps in {elapsed:.3f} s -> {ms_per_step:.2f} ms/step, loss {loss:.6g}")
+    log(f"{args.steps} steps in {elapsed:.3f} s -> {ms_per_step:.2f} ms/step, loss {loss:.10g}")
 
     kernels = {}
     for cls, (ms_sum, cnt) in tim.items():

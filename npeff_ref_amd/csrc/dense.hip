@@ -652,24 +652,27 @@ __global__ void __launch_bounds__(256)
     k_transpose(const float* __restrict__ in, int64_t rows, int64_t cols, float* __restrict__ out) {
   __shared__ float tile[32][33];
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-  const int64_t tiles_c = (cols + 31) / 32;
-  const int64_t tile_r = blockIdx.x / tiles_c, tile_c = blockIdx.x % tiles_c;
-  const int64_t r0 = tile_r * 32, c0 = tile_c * 32;
-  for (int i = ty; i < 32; i += 8) {
-    int64_t rr = r0 + i, cc = c0 + tx;
-    tile[i][tx] = (rr < rows && cc < cols) ? in[rr * cols + cc] : 0.0f;
-  }
-  __syncthreads();
-  for (int i = ty; i < 32; i += 8) {
-    int64_t cc = c0 + i, rr = r0 + tx;
-    if (cc < cols && rr < rows) out[cc * rows + rr] = tile[tx][i];
+  const int64_t tiles_c = (cols + 31) / 32, tiles_r = (rows + 31) / 32;
+  for (int64_t t = blockIdx.x; t < tiles_c * tiles_r; t += gridDim.x) {
+    const int64_t tile_r = t / tiles_c, tile_c = t % tiles_c;
+    const int64_t r0 = tile_r * 32, c0 = tile_c * 32;
+    for (int i = ty; i < 32; i += 8) {
+      int64_t rr = r0 + i, cc = c0 + tx;
+      tile[i][tx] = (rr < rows && cc < cols) ? in[rr * cols + cc] : 0.0f;
+    }
+    __syncthreads();
+    for (int i = ty; i < 32; i += 8) {
+      int64_t cc = c0 + i, rr = r0 + tx;
+      if (cc < cols && rr < rows) out[cc * rows + rr] = tile[tx][i];
+    }
+    __syncthreads();
   }
 }
 
 int launch_transpose(int64_t rows, int64_t cols, const float* in, float* out) {
   if (rows <= 0 || cols <= 0) return 0;
   int64_t tiles = ceil_div(rows, 32) * ceil_div(cols, 32);
-  DN_CHECK(tiles < (int64_t)INT32_MAX, "matrix too large for the transposition grid");
+  if (tiles > ((int64_t)1 << 22)) tiles = (int64_t)1 << 22;  // the kernel loops over the rest
   hipLaunchKernelGGL(k_transpose, dim3((unsigned)tiles), dim3(256), 0, stream(), in, rows, cols,
                      out);
   DN_LAUNCH_CHECK();

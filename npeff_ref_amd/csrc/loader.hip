@@ -188,9 +188,10 @@ int scan_long_cols(const int64_t* colptr, int64_t limit, int64_t n, int32_t* out
 // Loader kernels
 // ---------------------------------------------------------------------------
 
-__global__ void k_pef_rowptr(int64_t n_rows, int64_t k, int64_t* rowptr) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i <= n_rows) rowptr[i] = i * k;
+__global__ void __launch_bounds__(256) k_pef_rowptr(int64_t n_rows, int64_t k, int64_t* rowptr) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i <= n_rows; i += stride)
+    rowptr[i] = i * k;
 }
 
 // vals[e] /= (norms[row] + eps); one workgroup walks one row at a time.
@@ -216,27 +217,29 @@ __global__ void __launch_bounds__(256)
 __global__ void __launch_bounds__(256)
     k_build_maps(const int* __restrict__ count, int min_count, const int32_t* __restrict__ pos,
                  int64_t n_cols, int32_t* __restrict__ og_to_new, int32_t* __restrict__ new_to_og) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n_cols) return;
-  if (count[i] >= min_count) {
-    og_to_new[i] = pos[i];
-    new_to_og[pos[i]] = (int32_t)i;
-  } else {
-    og_to_new[i] = -1;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_cols; i += stride) {
+    if (count[i] >= min_count) {
+      og_to_new[i] = pos[i];
+      new_to_og[pos[i]] = (int32_t)i;
+    } else {
+      og_to_new[i] = -1;
+    }
   }
 }
 
 __global__ void __launch_bounds__(256) k_fill_i32(int32_t* p, int64_t n, int32_t v) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = v;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) p[i] = v;
 }
 
 // old_to_new[kept[i]] = i; for a column listed twice the last position wins,
 // as in the reference's sequential loop.
 __global__ void __launch_bounds__(256)
     k_retain_table(const int32_t* __restrict__ kept, int64_t n_kept, int32_t* __restrict__ table) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n_kept) atomicMax(&table[kept[i]], (int32_t)i);
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_kept; i += stride)
+    atomicMax(&table[kept[i]], (int32_t)i);
 }
 
 __global__ void __launch_bounds__(256)
@@ -265,8 +268,9 @@ __global__ void __launch_bounds__(256)
 
 __global__ void __launch_bounds__(256)
     k_remap_rowptr(int64_t* __restrict__ rowptr, int64_t n_rows, const int64_t* __restrict__ newpos) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i <= n_rows) rowptr[i] = newpos[rowptr[i]];
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i <= n_rows; i += stride)
+    rowptr[i] = newpos[rowptr[i]];
 }
 
 // One row of the stable transposition: entry e of this row goes to the next
@@ -289,9 +293,9 @@ __global__ void __launch_bounds__(256)
 __global__ void __launch_bounds__(256)
     k_collect_long(const int64_t* __restrict__ colptr, int64_t limit, int64_t n_cols,
                    const int32_t* __restrict__ pos, int32_t* __restrict__ long_cols) {
-  int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (j >= n_cols) return;
-  if (colptr[j + 1] - colptr[j] > limit) long_cols[pos[j]] = (int32_t)j;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x; j < n_cols; j += stride)
+    if (colptr[j + 1] - colptr[j] > limit) long_cols[pos[j]] = (int32_t)j;
 }
 
 __global__ void __launch_bounds__(256)
@@ -312,6 +316,8 @@ __global__ void __launch_bounds__(256)
   if (threadIdx.x == 0) partials[blockIdx.x] = sh[0];
 }
 
+// Grid of a grid-stride kernel over n items (every kernel launched with it loops); a launch is
+// limited to 2^32 threads in total, so grids are capped well below that.
 static unsigned grid_for(int64_t n, int64_t cap = 1 << 20) {
   int64_t g = ceil_div(n, 256);
   if (g < 1) g = 1;

@@ -10,6 +10,8 @@
 // reproducible run to run.
 #include "dnpeff_internal.hpp"
 
+#include <cstdlib>
+
 namespace dn {
 
 __device__ inline int bcast_i(int v, int src_lane) { return __builtin_amdgcn_readlane(v, src_lane); }
@@ -29,11 +31,12 @@ struct GatherDword {
   bool ok[VPL];
   int lane;
 
-  __device__ inline void init(int lane_, int r) {
+  // `width` components starting at the pointers given to run() and store()
+  __device__ inline void init(int lane_, int width) {
     lane = lane_;
 #pragma unroll
     for (int t = 0; t < VPL; t++) {
-      ok[t] = lane + 64 * t < r;
+      ok[t] = lane + 64 * t < width;
       acc[t] = 0.0f;
     }
   }
@@ -96,13 +99,14 @@ struct GatherVec4 {
   bool ok[T];
   int lane, sub, grp;
 
-  __device__ inline void init(int lane_, int r) {
+  // `width` components starting at the pointers given to run() and store()
+  __device__ inline void init(int lane_, int width) {
     lane = lane_;
     sub = lane % LPR;
     grp = lane / LPR;
 #pragma unroll
     for (int t = 0; t < T; t++) {
-      ok[t] = 4 * (sub + 64 * t) < r;
+      ok[t] = 4 * (sub + 64 * t) < width;
       acc[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
   }
@@ -230,47 +234,58 @@ __global__ void __launch_bounds__(256)
 
 // ---------------------------------------------------------------------------
 // T[j, :] = sum over column j's entries (ascending row) of val * W[row, :]
+//
+// The r components are cut into n_slices equal slices and workgroup b works on
+// slice b % n_slices.  Workgroups are handed to the 8 XCDs round-robin, so each
+// XCD only ever gathers from its own slice of W and that slice (n * r / n_slices
+// floats) stays in the XCD's 4 MB L2 instead of being evicted by the other half.
 // ---------------------------------------------------------------------------
 template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_short(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
-                   const float* __restrict__ tvals, int64_t m, int r, const float* __restrict__ W,
-                   float* __restrict__ T) {
+                   const float* __restrict__ tvals, int64_t m, int r, int n_slices,
+                   const float* __restrict__ W, float* __restrict__ T) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int64_t j = (int64_t)blockIdx.x * 4 + wave;
-  if (j >= m) return;
-  const int64_t p0 = colptr[j], p1 = colptr[j + 1];
-  if (p1 - p0 > SPMM_T_LONG) return;  // written by k_spmm_t_long
-  GT g;
-  g.init(lane, r);
-  g.run(rowind, tvals, p0, p1, W, r);
-  g.store(T + j * r);
+  const int slice = blockIdx.x % n_slices, width = r / n_slices;
+  // gridDim.x is a multiple of n_slices: the slice of a workgroup never changes
+  const int64_t group_stride = gridDim.x / n_slices;
+  for (int64_t grp = blockIdx.x / n_slices; grp * 4 < m; grp += group_stride) {
+    const int64_t j = grp * 4 + wave;
+    if (j >= m) break;
+    const int64_t p0 = colptr[j], p1 = colptr[j + 1];
+    if (p1 - p0 > SPMM_T_LONG) continue;  // written by k_spmm_t_long
+    GT g;
+    g.init(lane, width);
+    g.run(rowind, tvals, p0, p1, W + slice * width, r);
+    g.store(T + j * r + slice * width);
+  }
 }
 
 template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_long(const int32_t* __restrict__ long_cols, const int64_t* __restrict__ colptr,
                   const int32_t* __restrict__ rowind, const float* __restrict__ tvals, int r,
-                  const float* __restrict__ W, float* __restrict__ T) {
-  extern __shared__ __align__(16) float red_dyn[];  // [4][r]
+                  int n_slices, const float* __restrict__ W, float* __restrict__ T) {
+  extern __shared__ __align__(16) float red_dyn[];  // [4][width]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int64_t j = long_cols[blockIdx.x];
+  const int slice = blockIdx.x % n_slices, width = r / n_slices;
+  const int64_t j = long_cols[blockIdx.x / n_slices];
   const int64_t p0 = colptr[j], p1 = colptr[j + 1];
   const int64_t per = (((p1 - p0) + 3) / 4 + 63) / 64 * 64;  // quarter, rounded up to 64
   int64_t w0 = p0 + wave * per, w1 = w0 + per;
   if (w0 > p1) w0 = p1;
   if (w1 > p1) w1 = p1;
   GT g;
-  g.init(lane, r);
-  g.run(rowind, tvals, w0, w1, W, r);
-  g.store(red_dyn + wave * r);
+  g.init(lane, width);
+  g.run(rowind, tvals, w0, w1, W + slice * width, r);
+  g.store(red_dyn + wave * width);
   __syncthreads();
-  for (int c = threadIdx.x; c < r; c += 256) {
+  for (int c = threadIdx.x; c < width; c += 256) {
     float s = red_dyn[c];
-    s += red_dyn[r + c];
-    s += red_dyn[2 * r + c];
-    s += red_dyn[3 * r + c];
-    T[j * r + c] = s;
+    s += red_dyn[width + c];
+    s += red_dyn[2 * width + c];
+    s += red_dyn[3 * width + c];
+    T[j * r + slice * width + c] = s;
   }
 }
 
@@ -433,21 +448,40 @@ int launch_spmm_n_reduce(const dnpeff_csr* A, int r, const float* partials, floa
   return 0;
 }
 
+// Component slices for A^T W.  Measured on configs[1] (n = 10,000, r = 128): 1 slice 29 ms,
+// 2 slices 37 ms, 4 slices 64 ms -- re-reading the entries once per slice costs more than the
+// better L2 residency of W gains, so the default is 1.  DNPEFF_SPMM_T_SLICES = 2, 4 or 8
+// selects a sliced launch (for experiments on other shapes).
+static int spmm_t_slices(int64_t /*n*/, int r) {
+  if (const char* e = getenv("DNPEFF_SPMM_T_SLICES")) {
+    int v = atoi(e);
+    if ((v == 1 || v == 2 || v == 4 || v == 8) && r % v == 0 && (r / v) % 4 == 0) return v;
+  }
+  return 1;
+}
+
 int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   DN_CHECK(A->colptr != nullptr, "matrix has no transposed copy");
   if (A->n_cols == 0) return 0;
-  dim3 grid((unsigned)ceil_div(A->n_cols, 4)), block(256);
   const bool aligned = ((uintptr_t)T_mr % 16) == 0 && ((uintptr_t)W_nr % 16) == 0;
-  dispatch_gather(r, aligned, [&](auto tag) {
+  const int n_slices = (aligned && r % 4 == 0) ? spmm_t_slices(A->n_rows, r) : 1;
+  const int width = r / n_slices;
+  // one wave per (column, slice); a launch holds at most 2^32 threads, so beyond 2^23 workgroups
+  // each one loops over several column groups
+  int64_t wgs = ceil_div(A->n_cols, 4) * n_slices;
+  const int64_t max_wgs = ((int64_t)1 << 23) / n_slices * n_slices;
+  if (wgs > max_wgs) wgs = max_wgs;
+  dim3 grid((unsigned)wgs), block(256);
+  dispatch_gather(width, aligned, [&](auto tag) {
     using GT = typename decltype(tag)::type;
     hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), A->colptr, A->rowind,
-                       A->tvals, A->n_cols, r, W_nr, T_mr);
+                       A->tvals, A->n_cols, r, n_slices, W_nr, T_mr);
     if (A->n_long > 0) {
-      dim3 grid_l((unsigned)A->n_long);
-      const size_t lds = sizeof(float) * 4 * (size_t)r;
+      dim3 grid_l((unsigned)(A->n_long * n_slices));
+      const size_t lds = sizeof(float) * 4 * (size_t)width;
       hipLaunchKernelGGL((k_spmm_t_long<GT>), grid_l, block, lds, stream(), A->long_cols,
-                         A->colptr, A->rowind, A->tvals, r, W_nr, T_mr);
+                         A->colptr, A->rowind, A->tvals, r, n_slices, W_nr, T_mr);
     }
     return 0;
   });

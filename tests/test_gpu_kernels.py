@@ -138,3 +138,43 @@ def test_spsp_dense(r):
     assert _rel(hh.numpy(), orc.spsp_dense_f64(b, m, b, r)) < TOL
     A.close()
     B.close()
+
+
+@pytest.mark.parametrize("slices,r", [(2, 128), (4, 256), (8, 512), (4, 64)])
+def test_spmm_t_component_slices(slices, r, monkeypatch):
+    """The sliced launch of A^T W (one slice of the components per workgroup)."""
+    monkeypatch.setenv("DNPEFF_SPMM_T_SLICES", str(slices))
+    rng = np.random.default_rng(slices + r)
+    n, m = 3000, 30000
+    rowptr, colind, vals, _ = d.synth_pef_host(n, m, k_fixed=300, zipf_s=1.1, seed=7)
+    A = d.Csr.from_host(rowptr, colind, vals, m)
+    W = rng.random((n, r)).astype(np.float32)
+    dT = d.DeviceArray((m, r))
+    d.op_spmm_t(A, r, d.DeviceArray.from_numpy(W), dT)
+    T = dT.numpy()
+    want = orc.spmm_t_f64(rowptr, colind, vals, m, W)
+    # row-wise: short columns have small sums that a max-normalised check would hide
+    err = np.abs(T - want).max(axis=1) / (np.abs(want).max(axis=1) + 1e-300)
+    assert err.max() < TOL
+    A.close()
+
+
+def test_spmm_t_more_columns_than_one_pass_of_the_grid():
+    """36M columns: more (column, slice) work items than workgroups in the capped grid, so every
+    workgroup walks several column groups; columns without entries must come out as zeros."""
+    n, m, r = 64, 36_000_000, 16
+    rng = np.random.default_rng(3)
+    rp, ci, va = random_csr(rng, n, m, 500)
+    A = d.Csr.from_host(rp, ci, va, m)
+    W = rng.random((n, r)).astype(np.float32)
+    dT = d.DeviceArray((m, r))
+    d.op_init_uniform(0, m, r, 5, dT)  # stale contents that must all be overwritten
+    d.op_spmm_t(A, r, d.DeviceArray.from_numpy(W), dT)
+    T = dT.numpy()
+    used = np.unique(ci)
+    want = orc.spmm_t_f64(rp, ci, va, m, W)[used]
+    assert _rel(T[used], want) < TOL
+    mask = np.ones(m, dtype=bool)
+    mask[used] = False
+    assert not T[mask].any()
+    A.close()
