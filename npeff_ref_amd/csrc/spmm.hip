@@ -261,6 +261,97 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// Short and medium columns (at most SPMM_T_LONG entries), rank a multiple of 4: a wave owns
+// SPMM_T_COLS consecutive columns and each of its 64/LPR lane groups walks whole columns on its
+// own, so that a wave works on several columns at once, no cross-lane reduction is needed and
+// the column offsets of all its columns come from one coalesced load.  A group reads up to LPR
+// (row, value) pairs of its column with one load, hands them out with lane shuffles inside the
+// group and gathers each W row with one 16-byte load per lane; entries are applied in order.
+constexpr int SPMM_T_COLS = 32;
+
+template <int LPR, int T>
+__global__ void __launch_bounds__(256)
+    k_spmm_t_grouped(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
+                     const float* __restrict__ tvals, int64_t m, int r,
+                     const float* __restrict__ W, float* __restrict__ Tout) {
+  constexpr int G = 64 / LPR;
+  constexpr int UNR = T >= 4 ? 1 : T == 2 ? 2 : 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int sub = lane % LPR, grp = lane / LPR, gbase = grp * LPR;
+  const int64_t j0 = ((int64_t)blockIdx.x * 4 + wave) * SPMM_T_COLS;
+  if (j0 >= m) return;
+  bool ok[T];
+#pragma unroll
+  for (int t = 0; t < T; t++) ok[t] = 4 * (sub + 64 * t) < r;
+
+  // colptr[j0 + lane] for lane <= SPMM_T_COLS, as two 32-bit halves for the shuffles
+  const int64_t jc = j0 + lane < m ? j0 + lane : m;
+  const int64_t cp = lane <= SPMM_T_COLS ? colptr[jc] : 0;
+  const int cp_lo = (int)(uint32_t)(cp & 0xffffffffLL), cp_hi = (int)(cp >> 32);
+
+  for (int round = 0; round * G < SPMM_T_COLS; round++) {
+    const int jl = round * G + grp;
+    const int64_t j = j0 + jl;
+    const int64_t p0 = ((int64_t)__shfl(cp_hi, jl) << 32) | (uint32_t)__shfl(cp_lo, jl);
+    const int64_t p1 = ((int64_t)__shfl(cp_hi, jl + 1) << 32) | (uint32_t)__shfl(cp_lo, jl + 1);
+    const bool active = j < m && (p1 - p0) <= SPMM_T_LONG;  // longer ones: k_spmm_t_long
+    const int len = active ? (int)(p1 - p0) : 0;
+    float4 acc[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) acc[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+
+    for (int base = 0; __any(base < len); base += LPR) {
+      const int e = base + sub;
+      int my_i = 0;
+      float my_v = 0.0f;
+      if (e < len) {
+        my_i = rowind[p0 + e];
+        my_v = tvals[p0 + e];
+      }
+      const int cnt = len - base;  // entries of this group in the batch (may be <= 0 or > LPR)
+      // the wave walks to the largest count among its groups
+      int cmax = 0;
+#pragma unroll
+      for (int g = 0; g < G; g++) {
+        const int c = __builtin_amdgcn_readlane(cnt, g * LPR);
+        cmax = c > cmax ? c : cmax;
+      }
+      if (cmax > LPR) cmax = LPR;
+      for (int u = 0; u < cmax; u += UNR) {
+        float4 h[UNR][T];
+        float a[UNR];
+#pragma unroll
+        for (int uu = 0; uu < UNR; uu++) {
+          const int ue = u + uu;
+          const bool valid = ue < cnt && ue < LPR;
+          const int jrow = __shfl(my_i, gbase + (ue & (LPR - 1)));
+          a[uu] = __shfl(my_v, gbase + (ue & (LPR - 1)));
+          const float* x = W + (int64_t)jrow * r + 4 * sub;
+#pragma unroll
+          for (int t = 0; t < T; t++)
+            h[uu][t] = (valid && ok[t]) ? *reinterpret_cast<const float4*>(x + 256 * t)
+                                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          if (!valid) a[uu] = 0.0f;
+        }
+#pragma unroll
+        for (int uu = 0; uu < UNR; uu++)
+#pragma unroll
+          for (int t = 0; t < T; t++) {
+            acc[t].x = fmaf(a[uu], h[uu][t].x, acc[t].x);
+            acc[t].y = fmaf(a[uu], h[uu][t].y, acc[t].y);
+            acc[t].z = fmaf(a[uu], h[uu][t].z, acc[t].z);
+            acc[t].w = fmaf(a[uu], h[uu][t].w, acc[t].w);
+          }
+      }
+    }
+    if (active) {
+#pragma unroll
+      for (int t = 0; t < T; t++)
+        if (ok[t]) *reinterpret_cast<float4*>(Tout + j * r + 4 * (sub + 64 * t)) = acc[t];
+    }
+  }
+}
+
 template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_long(const int32_t* __restrict__ long_cols, const int64_t* __restrict__ colptr,
@@ -473,10 +564,27 @@ int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
   const int64_t max_wgs = ((int64_t)1 << 23) / n_slices * n_slices;
   if (wgs > max_wgs) wgs = max_wgs;
   dim3 grid((unsigned)wgs), block(256);
+  const bool grouped = aligned && r % 4 == 0 && n_slices == 1;
+  if (grouped) {
+    dim3 gg((unsigned)ceil_div(A->n_cols, 4 * SPMM_T_COLS));
+    const int r4 = r / 4;
+#define DN_GROUPED(LPR, T)                                                                     \
+  hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T>), gg, block, 0, stream(), A->colptr, A->rowind, \
+                     A->tvals, A->n_cols, r, W_nr, T_mr)
+    if (r4 <= 4) DN_GROUPED(4, 1);
+    else if (r4 <= 8) DN_GROUPED(8, 1);
+    else if (r4 <= 16) DN_GROUPED(16, 1);
+    else if (r4 <= 32) DN_GROUPED(32, 1);
+    else if (r4 <= 64) DN_GROUPED(64, 1);
+    else if (r4 <= 128) DN_GROUPED(64, 2);
+    else DN_GROUPED(64, 4);
+#undef DN_GROUPED
+  }
   dispatch_gather(width, aligned, [&](auto tag) {
     using GT = typename decltype(tag)::type;
-    hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), A->colptr, A->rowind,
-                       A->tvals, A->n_cols, r, n_slices, W_nr, T_mr);
+    if (!grouped)
+      hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), A->colptr, A->rowind,
+                         A->tvals, A->n_cols, r, n_slices, W_nr, T_mr);
     if (A->n_long > 0) {
       dim3 grid_l((unsigned)(A->n_long * n_slices));
       const size_t lds = sizeof(float) * 4 * (size_t)width;
