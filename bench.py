@@ -132,7 +132,9 @@ def main():
     nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=0, eps=args.eps, seed=args.seed))
     nmf.initialize()
     d.sync()
-    log(f"context (transposed CSR, factors) in {time.perf_counter() - t0:.1f} s")
+    n_dense, z_sparse = A.head_info()
+    log(f"context (dense head of {n_dense} columns, {z_sparse} entries stay sparse, transposed CSR, "
+        f"factors) in {time.perf_counter() - t0:.1f} s")
 
     # the CPU baseline starts from the same factors, so copy them before the GPU loop runs
     cpu = prepare_cpu_baseline(d, A, nmf, n, m, r, args.eps) if args.cpu_steps > 0 else None
@@ -190,7 +192,8 @@ def main():
         "config": {"workload": "configs[1] D-NPEFF NMF" if args.config == "c1" else args.config,
                    "n_examples": n, "n_features_full": cfg["m_full"], "n_features_kept": m,
                    "nnz": z, "nnz_per_row": cfg["k"], "zipf_s": cfg["s"], "rank": r,
-                   "eps": args.eps, "seed": args.seed},
+                   "eps": args.eps, "seed": args.seed, "dense_head_columns": n_dense,
+                   "nnz_sparse_part": z_sparse},
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "kernels": kernels,

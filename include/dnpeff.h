@@ -125,6 +125,22 @@ int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out);
  * replacement of CsrTranspose (cc/cuda_d_npeff/src/cuda/ops/transpose.h:170-439). */
 int dnpeff_csr_build_transpose(dnpeff_csr* A);
 
+/* Split off the dense head: every column held by at least ceil(min_fill * n_rows) rows
+ * leaves the sparse structures and is stored as a dense block, so that its share of A H^T and
+ * A^T W runs as a matrix product on the matrix cores; the other entries stay sparse.  The
+ * products of the split matrix are the same sums in another order; they then need a rank that
+ * is a multiple of 4.  dnpeff_csr_download and the loader calls still see the whole matrix;
+ * any call that edits the matrix undoes the split.  The threshold is raised until both dense
+ * blocks fit an eighth of the device memory.  min_fill <= 0 removes the split.  n_dense (may
+ * be NULL) receives the number of columns in the head.
+ * No counterpart in the reference, which hands the whole matrix to cusparseSpMM
+ * (device_contexts1.h:255-265); dnpeff_nmf_create applies it by itself (fill 1/16, rank >= 64
+ * and a multiple of 4, at least 1024 rows) unless the caller has split the matrix already. */
+int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* n_dense);
+
+/* Columns in the dense head (0 = not split) and entries left in the sparse part. */
+int dnpeff_csr_head_info(const dnpeff_csr* A, int64_t* n_dense, int64_t* nnz_sparse);
+
 /* Copy the transposed CSR back: colptr[n_cols+1], rowind[nnz], vals[nnz]. */
 int dnpeff_csr_download_transpose(dnpeff_csr* A, int64_t* colptr, int32_t* rowind, float* vals);
 

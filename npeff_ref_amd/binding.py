@@ -60,6 +60,8 @@ SIGNATURES = {
     "dnpeff_csr_kept_indices": (C.c_int, [_p, _p]),
     "dnpeff_csr_sq_norm": (C.c_int, [_p, C.POINTER(_f64)]),
     "dnpeff_csr_build_transpose": (C.c_int, [_p]),
+    "dnpeff_csr_split_dense_head": (C.c_int, [_p, C.c_double, C.POINTER(C.c_int64)]),
+    "dnpeff_csr_head_info": (C.c_int, [_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "dnpeff_csr_download_transpose": (C.c_int, [_p, _p, _p, _p]),
     "dnpeff_csr_release": (C.c_int, [_p, C.c_int]),
     "dnpeff_csr_destroy": (C.c_int, [_p]),
@@ -345,6 +347,18 @@ class Csr:
         v = _f64(0)
         _check(lib.dnpeff_csr_sq_norm(self._h, C.byref(v)))
         return v.value
+
+    def split_dense_head(self, min_fill: float) -> int:
+        """Moves the columns held by at least min_fill of the rows into a dense block
+        (min_fill <= 0 undoes it); returns the number of such columns."""
+        nd = _i64(0)
+        _check(lib.dnpeff_csr_split_dense_head(self._h, float(min_fill), C.byref(nd)))
+        return nd.value
+
+    def head_info(self):
+        nd, zs = _i64(0), _i64(0)
+        _check(lib.dnpeff_csr_head_info(self._h, C.byref(nd), C.byref(zs)))
+        return nd.value, zs.value
 
     def build_transpose(self):
         _check(lib.dnpeff_csr_build_transpose(self._h))

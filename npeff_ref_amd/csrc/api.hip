@@ -3,6 +3,7 @@
 #include "dnpeff_internal.hpp"
 
 #include <cmath>
+#include <cstdlib>
 #include <utility>
 #include <vector>
 
@@ -99,6 +100,24 @@ DN_API int dnpeff_nmf_destroy(dnpeff_nmf* nmf) {
   return 0;
 }
 
+// Splits off the dense head when the products can use it: rank a multiple of 4 and at least 64
+// (below that a column of the dense block costs more than its entries do as gathers), enough
+// rows for the fill fraction to mean something.  A column goes to the head when at least 1/16 of
+// the rows hold it; DNPEFF_DENSE_FILL overrides the fraction (0 = never split).
+static int default_head_split(dnpeff_csr* A, int rank) {
+  double fill = 1.0 / 16.0;
+  if (const char* e = getenv("DNPEFF_DENSE_FILL")) fill = atof(e);
+  if (A->tail) {
+    if (rank % 4 == 0) return 0;  // split by the caller: keep it
+    fill = 0.0;
+  }
+  if (fill <= 0.0 || fill > 1.0 || rank % 4 != 0 || rank < 64 || A->n_rows < 1024) {
+    if (A->tail) return dnpeff_csr_split_dense_head(A, 0.0, nullptr);
+    return 0;
+  }
+  return dnpeff_csr_split_dense_head(A, fill, nullptr);
+}
+
 DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out) {
   clear_error();
   DN_CHECK(out != nullptr, "out is NULL");
@@ -107,8 +126,8 @@ DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, d
   DN_CHECK(rank >= 1 && rank <= 1024, "rank %d outside [1, 1024]", rank);
   // multi_mu_dense_factors_nmf1.h:95-99
   DN_CHECK(A->n_rows <= A->n_cols, "Error: Not handling matrices with more rows than columns yet.");
-  DN_TRY(dnpeff_csr_build_transpose(A));
-  DN_TRY(csr_ensure_partials(A, rank));
+  DN_TRY(default_head_split(A, rank));
+  DN_TRY(csr_ensure_products(A, rank));
   dnpeff_nmf* h = new dnpeff_nmf();
   h->A = A; h->r = rank; h->eps = eps; h->seed = (uint64_t)seed;
   h->n = A->n_rows; h->m = A->n_cols;
@@ -152,10 +171,10 @@ DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
   DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N));
-  DN_TRY(launch_spmm_n(A, h->r, h->H, h->Nw, A->partials));
+  DN_TRY(launch_spmm_n(A, h->r, h->H));
   DN_TRY(h->prof.end());
   DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N_REDUCE));
-  DN_TRY(launch_spmm_n_reduce(A, h->r, A->partials, h->Nw));
+  DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
   DN_TRY(h->prof.end());
   DN_TRY(h->prof.begin(DNPEFF_K_GRAM_H));
   DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
@@ -198,8 +217,8 @@ DN_API int dnpeff_nmf_loss_terms(dnpeff_nmf* h, double* sq_norm_A, double* pos, 
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
   // neg = <W^T A, H> = <A H^T, W>
-  DN_TRY(launch_spmm_n(A, h->r, h->H, h->Nw, A->partials));
-  DN_TRY(launch_spmm_n_reduce(A, h->r, A->partials, h->Nw));
+  DN_TRY(launch_spmm_n(A, h->r, h->H));
+  DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
   DN_TRY(launch_dot(h->n * h->r, h->Nw, h->W, h->dot_ws, h->dot_ws + DOT_BLOCKS));
   // pos = <H, (W^T W) H> = <W^T W, H H^T>
   DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));

@@ -100,10 +100,25 @@ int launch_transpose(int64_t rows, int64_t cols, const float* in, float* out);
 // ---- sparse kernels (spmm.hip) ----
 constexpr int64_t SPMM_N_CHUNK = 2048;  // entries of one row handled by one workgroup
 constexpr int64_t SPMM_T_LONG = 256;    // columns longer than this get a whole workgroup
-int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr, float* N_nr, float* partials);
-int launch_spmm_n_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr);
+// A H^T in two steps (partial sums, then their reduction); both cover the sparse part and the
+// dense head of A.  Need csr_ensure_products(A, r).
+int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr);
+int launch_spmm_n_reduce(const dnpeff_csr* A, int r, float* N_nr);
 int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials);
+int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr);
+
+// Columns present in many rows, held as a dense block in both orientations (head.hip).
+struct dense_head {
+  int64_t n_d = 0;      // columns in the head
+  int64_t n_d_pad = 0;  // n_d rounded up to 128
+  int64_t n_pad = 0;    // rows rounded up to 128
+  int32_t* cols = nullptr;  // [n_d] column of each head slot, ascending
+  float* cm = nullptr;      // [n_d_pad, n_pad]: cm[k * n_pad + i] = A[i, cols[k]]
+  float* rm = nullptr;      // [n_pad, n_d_pad]: rm[i * n_d_pad + k] = A[i, cols[k]]
+  float* ws = nullptr;      // gathered factor rows + slice partials of the products
+  int64_t ws_floats = 0;
+};
 
 }  // namespace dn
 
@@ -129,9 +144,22 @@ struct dnpeff_csr {
   // workspace for the per-chunk partial sums of A H^T ([n_chunks, r])
   float* partials = nullptr;
   int64_t partials_floats = 0;
+  // after dnpeff_csr_split_dense_head: the dense block and the matrix of the remaining entries
+  // (same shape, owned), which carries the derived structures the products use
+  dn::dense_head head;
+  dnpeff_csr* tail = nullptr;
 };
 
 namespace dn {
+inline dnpeff_csr* sparse_part(dnpeff_csr* A) { return A->tail ? A->tail : A; }
+inline const dnpeff_csr* sparse_part(const dnpeff_csr* A) { return A->tail ? A->tail : A; }
 int csr_ensure_chunks(dnpeff_csr* A);
 int csr_ensure_partials(dnpeff_csr* A, int r);
+// Everything A H^T and A^T W at rank r need: transposed copy and work lists of the sparse part,
+// workspaces of the sparse part and of the dense head.
+int csr_ensure_products(dnpeff_csr* A, int r);
+int head_ensure_workspace(dnpeff_csr* A, int r);
+int launch_head_n(const dnpeff_csr* A, int r, const float* H_mr);
+int launch_head_n_add(const dnpeff_csr* A, int r, float* N_nr);
+int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 }  // namespace dn

@@ -1,0 +1,308 @@
+// Dense head of a sparse matrix: the columns that are present in a sizeable fraction of the
+// rows are taken out of the CSR structures and kept as a dense block, in both orientations.
+// Their share of A H^T and A^T W is then a matrix product on fp32 MFMA (32x32x2) instead of one
+// 4r-byte gather per entry; the remaining ("tail") entries stay sparse.
+//
+//   A H^T  = tail(A) H^T + D  Hd        D  [n, n_d] dense block, Hd = rows of H of the head
+//   A^T W  : rows of the head  = D^T W, all other rows = tail(A)^T W
+//
+// Both products have the form C = P^T Q with P [K, ldp] and Q [K, r] sharing the contraction
+// index K as their slow index: P = D^T ("cm", K = n_d) for the first, P = D ("rm", K = n) for
+// the second.
+#include "dnpeff_internal.hpp"
+
+#include <type_traits>
+
+namespace dn {
+
+typedef float acc16 __attribute__((ext_vector_type(16)));
+
+// ---------------------------------------------------------------------------
+// C[slice] = P[k in slice]^T Q[k in slice]
+//
+// A workgroup of 4 waves owns a 128 x 128 tile of C and a contiguous range of K, streamed in
+// tiles of 32 contraction rows through two LDS slots (P tile then Q tile, 16 KB each), fetched
+// with 16-byte loads two tiles ahead into registers.  v_mfma_f32_32x32x2f32 takes from lane l
+// A[i = l%32][k = l/32] and B[k = l/32][j = l%32]; the 32 rows (columns) of an operand block are
+// every fourth element of the 128-wide tile (block a holds 4 i + a), stored in LDS as four runs
+// of 32 floats, so one 16-byte global load feeds four blocks and every LDS read is conflict
+// free.  Wave (wm, wn) owns blocks {2 wm, 2 wm + 1} x {2 wn, 2 wn + 1}.
+// ---------------------------------------------------------------------------
+constexpr int PTQ_KB = 32;
+constexpr int PTQ_HALF = PTQ_KB * 128;   // floats of one operand tile
+constexpr int PTQ_SLOT = 2 * PTQ_HALF;   // floats of one slot
+
+struct PtqStage {
+  float4 p[4], q[4];
+};
+
+__global__ void __launch_bounds__(256)
+    k_ptq(const float* __restrict__ P, int64_t ldp, int64_t K, const float* __restrict__ Q, int r,
+          int64_t M, int64_t M_pad, int64_t tiles_per_slice, float* __restrict__ out) {
+  extern __shared__ __align__(16) float lds[];  // 2 * PTQ_SLOT floats
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t m0 = (int64_t)blockIdx.x * 128;
+  const int n0 = blockIdx.y * 128;
+  const int64_t all_tiles = (K + PTQ_KB - 1) / PTQ_KB;
+  const int64_t t0 = (int64_t)blockIdx.z * tiles_per_slice;
+  int64_t n_tiles = all_tiles - t0;
+  if (n_tiles > tiles_per_slice) n_tiles = tiles_per_slice;
+  if (n_tiles < 0) n_tiles = 0;
+
+  // loader role of a thread: 16-byte column li of rows lr + 8 q of a tile
+  const int li = threadIdx.x & 31, lr = threadIdx.x >> 5;
+  const bool qcol_ok = n0 + 4 * li < r;
+  const float* pP = P + m0 + 4 * li;
+  const float* pQ = Q + n0 + 4 * li;
+
+  auto fetch = [&](PtqStage& s, int64_t tile) {
+    const int64_t kbase = (t0 + tile) * PTQ_KB + lr;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int64_t k = kbase + 8 * q;
+      const bool ok = tile < n_tiles && k < K;
+      s.p[q] = ok ? *reinterpret_cast<const float4*>(pP + k * ldp)
+                  : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      s.q[q] = (ok && qcol_ok) ? *reinterpret_cast<const float4*>(pQ + k * (int64_t)r)
+                               : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  auto commit = [&](const PtqStage& s, float* slot) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      float* a = slot + (lr + 8 * q) * 128 + li;
+      a[0] = s.p[q].x; a[32] = s.p[q].y; a[64] = s.p[q].z; a[96] = s.p[q].w;
+      float* b = a + PTQ_HALF;
+      b[0] = s.q[q].x; b[32] = s.q[q].y; b[64] = s.q[q].z; b[96] = s.q[q].w;
+    }
+  };
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+  auto mfma_slot = [&](const float* slot) {
+    const float* pa = slot + half * 128 + 64 * wm + l32;
+    const float* pb = slot + PTQ_HALF + half * 128 + 64 * wn + l32;
+    constexpr int GRP = 4;
+#pragma unroll
+    for (int g = 0; g < PTQ_KB / 2; g += GRP) {
+      float xa[GRP][2], xb[GRP][2];
+#pragma unroll
+      for (int u = 0; u < GRP; u++) {
+        xa[u][0] = pa[2 * (g + u) * 128];
+        xa[u][1] = pa[2 * (g + u) * 128 + 32];
+        xb[u][0] = pb[2 * (g + u) * 128];
+        xb[u][1] = pb[2 * (g + u) * 128 + 32];
+      }
+#pragma unroll
+      for (int u = 0; u < GRP; u++)
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u][i], xb[u][j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  PtqStage s0, s1;
+  fetch(s0, 0);
+  fetch(s1, 1);
+  if (n_tiles > 0) commit(s0, lds);
+  __syncthreads();
+  // iteration t: tile t sits in slot t & 1; its register stage is free and receives tile t + 2;
+  // tile t + 1 moves from the other stage to the other slot after the MFMAs
+  int64_t t = 0;
+  for (; t + 2 <= n_tiles; t += 2) {
+    fetch(s0, t + 2);
+    mfma_slot(lds);
+    commit(s1, lds + PTQ_SLOT);
+    __syncthreads();
+    fetch(s1, t + 3);
+    mfma_slot(lds + PTQ_SLOT);
+    if (t + 2 < n_tiles) commit(s0, lds);
+    __syncthreads();
+  }
+  if (t < n_tiles) mfma_slot(lds);
+
+  // D layout of a 32x32 block: reg v of lane l holds row 8 (v/4) + 4 (l/32) + v%4, column l%32;
+  // block (a, b) row ib is C row 4 ib + a, column jb is C column 4 jb + b.  The wave's two
+  // column blocks are adjacent columns: one 8-byte store.
+  const int n = 4 * l32 + 2 * wn;
+  if (n0 + n < r) {
+    float* base = out + ((int64_t)blockIdx.z * M_pad + m0) * r + n0 + n;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int ib = 8 * (v >> 2) + 4 * half + (v & 3);
+        const int m = 4 * ib + 2 * wm + i;
+        if (m0 + m < M)
+          *reinterpret_cast<float2*>(base + (int64_t)m * r) = make_float2(acc[i][0][v], acc[i][1][v]);
+      }
+  }
+}
+
+// slices of K so that the launch holds about a thousand workgroups
+static int64_t ptq_slices(int64_t tiles_mn, int64_t k_tiles) {
+  int64_t s = 1024 / (tiles_mn > 0 ? tiles_mn : 1);
+  if (s > 64) s = 64;
+  if (s > k_tiles) s = k_tiles;
+  return s < 1 ? 1 : s;
+}
+
+static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, int r, int64_t M,
+                      int64_t M_pad, int64_t slices, float* out) {
+  static bool attr_set = false;
+  const size_t lds = sizeof(float) * 2 * PTQ_SLOT;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_ptq),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int64_t k_tiles = ceil_div(K, PTQ_KB);
+  const int64_t per = ceil_div(k_tiles, slices);
+  DN_CHECK(M_pad % 128 == 0 && ldp % 4 == 0 && r % 4 == 0, "dense product: misaligned operands");
+  DN_CHECK(M_pad / 128 < ((int64_t)1 << 22), "dense product: too many row tiles");
+  dim3 grid((unsigned)(M_pad / 128), (unsigned)ceil_div(r, 128), (unsigned)slices);
+  hipLaunchKernelGGL(k_ptq, grid, dim3(256), lds, stream(), P, ldp, K, Q, r, M, M_pad, per, out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+// Hd[k] = H[cols[k]]
+__global__ void __launch_bounds__(256)
+    k_head_gather(const float* __restrict__ H, const int32_t* __restrict__ cols, int64_t n_d, int r,
+                  float* __restrict__ Hd) {
+  const int r4 = r >> 2;
+  const int64_t total = n_d * r4, stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int64_t k = e / r4;
+    const int c = (int)(e % r4);
+    reinterpret_cast<float4*>(Hd + k * r)[c] =
+        reinterpret_cast<const float4*>(H + (int64_t)cols[k] * r)[c];
+  }
+}
+
+// N[i] += sum over slices of ws[s][i]   (slices summed in fp64, in slice order)
+__global__ void __launch_bounds__(256)
+    k_head_add(const float* __restrict__ ws, int64_t slices, int64_t rows, int64_t rows_pad, int r,
+               float* __restrict__ N) {
+  const int r4 = r >> 2;
+  const int64_t total = rows * r4, stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int64_t i = e / r4;
+    const int c = (int)(e % r4);
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+    for (int64_t s = 0; s < slices; s++) {
+      const float4 v = reinterpret_cast<const float4*>(ws + (s * rows_pad + i) * r)[c];
+      s0 += v.x; s1 += v.y; s2 += v.z; s3 += v.w;
+    }
+    float4* o = reinterpret_cast<float4*>(N + i * r) + c;
+    float4 cur = *o;
+    cur.x = (float)((double)cur.x + s0);
+    cur.y = (float)((double)cur.y + s1);
+    cur.z = (float)((double)cur.z + s2);
+    cur.w = (float)((double)cur.w + s3);
+    *o = cur;
+  }
+}
+
+// T[cols[k]] = sum over slices of ws[s][k]
+__global__ void __launch_bounds__(256)
+    k_head_scatter(const float* __restrict__ ws, int64_t slices, int64_t n_d, int64_t n_d_pad, int r,
+                   const int32_t* __restrict__ cols, float* __restrict__ T) {
+  const int r4 = r >> 2;
+  const int64_t total = n_d * r4, stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int64_t k = e / r4;
+    const int c = (int)(e % r4);
+    float4 out;
+    if (slices == 1) {
+      out = reinterpret_cast<const float4*>(ws + k * r)[c];
+    } else {
+      double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+      for (int64_t s = 0; s < slices; s++) {
+        const float4 v = reinterpret_cast<const float4*>(ws + (s * n_d_pad + k) * r)[c];
+        s0 += v.x; s1 += v.y; s2 += v.z; s3 += v.w;
+      }
+      out = make_float4((float)s0, (float)s1, (float)s2, (float)s3);
+    }
+    reinterpret_cast<float4*>(T + (int64_t)cols[k] * r)[c] = out;
+  }
+}
+
+static unsigned elem_grid(int64_t count) {
+  int64_t g = ceil_div(count, 256);
+  if (g > (1 << 20)) g = 1 << 20;
+  return (unsigned)(g < 1 ? 1 : g);
+}
+
+static int64_t head_slices_n(const dense_head& h, int r) {
+  return ptq_slices((h.n_pad / 128) * ceil_div(r, 128), ceil_div(h.n_d, PTQ_KB));
+}
+static int64_t head_slices_t(const dense_head& h, int r, int64_t n) {
+  return ptq_slices((h.n_d_pad / 128) * ceil_div(r, 128), ceil_div(n, PTQ_KB));
+}
+
+int head_ensure_workspace(dnpeff_csr* A, int r) {
+  dense_head& h = A->head;
+  if (h.n_d == 0) return 0;
+  DN_CHECK(r % 4 == 0, "a matrix with a dense head needs a rank that is a multiple of 4 (got %d)", r);
+  const int64_t gather = h.n_d_pad * r;
+  const int64_t wn = head_slices_n(h, r) * h.n_pad * r;
+  const int64_t wt = head_slices_t(h, r, A->n_rows) * h.n_d_pad * r;
+  const int64_t need = gather + (wn > wt ? wn : wt);
+  if (h.ws && h.ws_floats >= need) return 0;
+  dfree(h.ws);
+  h.ws = nullptr;
+  DN_TRY(dmalloc(&h.ws, need));
+  h.ws_floats = need;
+  return 0;
+}
+
+// slice partials of D Hd into the workspace
+int launch_head_n(const dnpeff_csr* A, int r, const float* H_mr) {
+  const dense_head& h = A->head;
+  if (h.n_d == 0) return 0;
+  DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)H_mr % 16) == 0, "dense head: workspace or alignment");
+  float* Hd = h.ws;
+  float* part = h.ws + h.n_d_pad * r;
+  hipLaunchKernelGGL(k_head_gather, dim3(elem_grid(h.n_d * (r / 4))), dim3(256), 0, stream(), H_mr,
+                     h.cols, h.n_d, r, Hd);
+  return launch_ptq(h.cm, h.n_pad, h.n_d, Hd, r, A->n_rows, h.n_pad, head_slices_n(h, r), part);
+}
+
+// N += D Hd from the slice partials
+int launch_head_n_add(const dnpeff_csr* A, int r, float* N_nr) {
+  const dense_head& h = A->head;
+  if (h.n_d == 0) return 0;
+  const float* part = h.ws + h.n_d_pad * r;
+  hipLaunchKernelGGL(k_head_add, dim3(elem_grid(A->n_rows * (r / 4))), dim3(256), 0, stream(), part,
+                     head_slices_n(h, r), A->n_rows, h.n_pad, r, N_nr);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+// rows of the head of A^T W (overwrites what the sparse kernels stored there)
+int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
+  const dense_head& h = A->head;
+  if (h.n_d == 0) return 0;
+  DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)W_nr % 16) == 0 && ((uintptr_t)T_mr % 16) == 0,
+           "dense head: workspace or alignment");
+  float* part = h.ws + h.n_d_pad * r;
+  const int64_t slices = head_slices_t(h, r, A->n_rows);
+  DN_TRY(launch_ptq(h.rm, h.n_d_pad, A->n_rows, W_nr, r, h.n_d, h.n_d_pad, slices, part));
+  hipLaunchKernelGGL(k_head_scatter, dim3(elem_grid(h.n_d * (r / 4))), dim3(256), 0, stream(), part,
+                     slices, h.n_d, h.n_d_pad, r, h.cols, T_mr);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace dn

@@ -3,6 +3,8 @@
 // with the reference's host code; see include/dnpeff.h for the citations.
 #include "dnpeff_internal.hpp"
 
+#include <cmath>
+
 #include <cstdarg>
 #include <cstring>
 #include <vector>
@@ -228,6 +230,32 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// table[c] = -1 for the columns of the head, c for the others
+__global__ void __launch_bounds__(256)
+    k_tail_table(const int32_t* __restrict__ og_to_new, int64_t n_cols, int32_t* __restrict__ table) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_cols; i += stride)
+    table[i] = og_to_new[i] >= 0 ? -1 : (int32_t)i;
+}
+
+// Entries of the head's columns into both dense blocks; a workgroup per row.  Entries that
+// repeat a (row, column) pair add up, as they do in the sparse products.
+__global__ void __launch_bounds__(256)
+    k_head_fill(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
+                const float* __restrict__ vals, int64_t n_rows, const int32_t* __restrict__ slot_of,
+                float* __restrict__ cm, int64_t n_pad, float* __restrict__ rm, int64_t n_d_pad) {
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    const int64_t e1 = rowptr[row + 1];
+    for (int64_t e = rowptr[row] + threadIdx.x; e < e1; e += 256) {
+      const int32_t k = slot_of[colind[e]];
+      if (k >= 0) {
+        atomicAdd(&cm[(int64_t)k * n_pad + row], vals[e]);
+        atomicAdd(&rm[row * n_d_pad + k], vals[e]);
+      }
+    }
+  }
+}
+
 __global__ void __launch_bounds__(256) k_fill_i32(int32_t* p, int64_t n, int32_t v) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) p[i] = v;
@@ -360,7 +388,17 @@ static int apply_column_table(dnpeff_csr* A, const int32_t* table, int64_t new_n
   return 0;
 }
 
+static void drop_head(dnpeff_csr* A) {
+  if (A->tail) {
+    dnpeff_csr_destroy(A->tail);
+    A->tail = nullptr;
+  }
+  dfree(A->head.cols); dfree(A->head.cm); dfree(A->head.rm); dfree(A->head.ws);
+  A->head = dense_head();
+}
+
 static void drop_derived(dnpeff_csr* A) {
+  drop_head(A);
   dfree(A->colptr); A->colptr = nullptr;
   dfree(A->rowind); A->rowind = nullptr;
   dfree(A->tvals); A->tvals = nullptr;
@@ -377,6 +415,13 @@ int csr_ensure_chunks(dnpeff_csr* A) {
   DN_HIP(hipMemcpy(&A->n_chunks, A->chunk_base + A->n_rows, sizeof(int64_t),
                    hipMemcpyDeviceToHost));
   return 0;
+}
+
+int csr_ensure_products(dnpeff_csr* A, int r) {
+  dnpeff_csr* S = sparse_part(A);
+  DN_TRY(dnpeff_csr_build_transpose(S));
+  DN_TRY(csr_ensure_partials(S, r));
+  return head_ensure_workspace(A, r);
 }
 
 int csr_ensure_partials(dnpeff_csr* A, int r) {
@@ -692,6 +737,98 @@ DN_API int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out) {
   double s = 0.0;
   for (int i = 0; i < blocks; i++) s += h[i];
   *out = s;
+  return 0;
+}
+
+DN_API int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* n_dense) {
+  clear_error();
+  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(min_fill <= 1.0, "min_fill %g above 1", min_fill);
+  hipStream_t st = stream();
+  drop_derived(A);
+  if (n_dense) *n_dense = 0;
+  if (min_fill <= 0.0) return 0;
+  const int64_t m = A->n_cols, n = A->n_rows;
+  if (m == 0 || n == 0 || A->nnz == 0) return 0;
+  int64_t thr = (int64_t)ceil(min_fill * (double)n);
+  if (thr < 1) thr = 1;
+  int* count = nullptr;
+  int32_t *pos = nullptr, *slot_of = nullptr, *cols = nullptr, *table = nullptr;
+  DN_TRY(dmalloc(&count, m));
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)m, st));
+  hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
+                     count);
+  DN_LAUNCH_CHECK();
+  DN_TRY(dmalloc(&pos, m + 1));
+  // both dense blocks together stay below an eighth of the device memory: raise the bar
+  // until they do
+  size_t free_b = 0, total_b = 0;
+  DN_HIP(hipMemGetInfo(&free_b, &total_b));
+  const int64_t n_pad = ceil_div(n, 128) * 128;
+  int32_t n_d = 0;
+  for (;;) {
+    DN_CHECK(thr <= (int64_t)INT32_MAX, "dense head: threshold overflow");
+    DN_TRY(scan_keep_mask(count, (int)thr, m, pos));
+    DN_HIP(hipMemcpy(&n_d, pos + m, sizeof(int32_t), hipMemcpyDeviceToHost));
+    const double bytes = 2.0 * 4.0 * (double)n_pad * (double)(ceil_div(n_d, 128) * 128);
+    if (bytes <= (double)total_b / 8.0 || thr > n) break;
+    thr *= 2;
+  }
+  if (n_d == 0 || thr > n) {
+    dfree(count); dfree(pos);
+    return 0;
+  }
+  const int64_t n_d_pad = ceil_div(n_d, 128) * 128;
+  int s = dmalloc(&slot_of, m) || dmalloc(&cols, (int64_t)n_d) || dmalloc(&table, m);
+  if (!s) {
+    hipLaunchKernelGGL(k_build_maps, dim3(grid_for(m)), dim3(256), 0, st, count, (int)thr, pos, m,
+                       slot_of, cols);
+    hipLaunchKernelGGL(k_tail_table, dim3(grid_for(m)), dim3(256), 0, st, slot_of, m, table);
+  }
+  dense_head& h = A->head;
+  if (!s) s = dmalloc(&h.cm, n_d_pad * n_pad) || dmalloc(&h.rm, n_pad * n_d_pad);
+  if (!s && (hipMemsetAsync(h.cm, 0, sizeof(float) * (size_t)(n_d_pad * n_pad), st) != hipSuccess ||
+             hipMemsetAsync(h.rm, 0, sizeof(float) * (size_t)(n_pad * n_d_pad), st) != hipSuccess)) {
+    set_error("dense head: clearing the blocks failed");
+    s = 1;
+  }
+  if (!s) {
+    hipLaunchKernelGGL(k_head_fill, dim3(grid_for(n * 256)), dim3(256), 0, st, A->rowptr, A->colind,
+                       A->vals, n, slot_of, h.cm, n_pad, h.rm, n_d_pad);
+    if (hipGetLastError() != hipSuccess) { set_error("dense head: launch failed"); s = 1; }
+  }
+  // the remaining entries: a copy of the row-major arrays without the head's columns
+  dnpeff_csr* T = nullptr;
+  if (!s) {
+    T = new dnpeff_csr();
+    T->n_rows = n; T->n_cols = m; T->nnz = A->nnz; T->full_dense_size = A->full_dense_size;
+    s = dmalloc(&T->rowptr, n + 1) || dmalloc(&T->colind, A->nnz) || dmalloc(&T->vals, A->nnz);
+    if (!s && (hipMemcpyAsync(T->rowptr, A->rowptr, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToDevice, st) != hipSuccess ||
+               hipMemcpyAsync(T->colind, A->colind, sizeof(int32_t) * A->nnz, hipMemcpyDeviceToDevice, st) != hipSuccess ||
+               hipMemcpyAsync(T->vals, A->vals, sizeof(float) * A->nnz, hipMemcpyDeviceToDevice, st) != hipSuccess)) {
+      set_error("dense head: copying the entries failed");
+      s = 1;
+    }
+    if (!s) s = apply_column_table(T, table, m);
+  }
+  (void)hipStreamSynchronize(st);
+  dfree(count); dfree(pos); dfree(slot_of); dfree(table);
+  if (s) {
+    if (T) dnpeff_csr_destroy(T);
+    dfree(cols);
+    drop_head(A);
+    return s;
+  }
+  h.n_d = n_d; h.n_d_pad = n_d_pad; h.n_pad = n_pad; h.cols = cols;
+  A->tail = T;
+  if (n_dense) *n_dense = n_d;
+  return 0;
+}
+
+DN_API int dnpeff_csr_head_info(const dnpeff_csr* A, int64_t* n_dense, int64_t* nnz_sparse) {
+  DN_CHECK(A != nullptr, "matrix is NULL");
+  if (n_dense) *n_dense = A->head.n_d;
+  if (nnz_sparse) *nnz_sparse = sparse_part(A)->nnz;
   return 0;
 }
 

@@ -514,9 +514,12 @@ static int dispatch_gather(int r, bool aligned16, F&& f) {
   }
 }
 
-int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr, float* /*N_nr*/, float* partials) {
+int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
-  DN_CHECK(A->rowptr && A->chunk_base, "matrix has no row-major copy / work list");
+  DN_TRY(launch_head_n(A_full, r, H_mr));
+  const dnpeff_csr* A = sparse_part(A_full);
+  float* partials = A->partials;
+  DN_CHECK(A->rowptr && A->chunk_base && partials, "matrix has no row-major copy / work list");
   if (A->n_chunks == 0) return 0;
   DN_CHECK(A->n_chunks < (int64_t)INT32_MAX, "too many work chunks");
   dim3 grid((unsigned)A->n_chunks), block(256);
@@ -531,7 +534,13 @@ int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr, float* /*N_nr*/
   return 0;
 }
 
-int launch_spmm_n_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr) {
+int launch_spmm_n_reduce(const dnpeff_csr* A_full, int r, float* N_nr) {
+  const dnpeff_csr* A = sparse_part(A_full);
+  DN_TRY(launch_chunk_reduce(A, r, A->partials, N_nr));
+  return launch_head_n_add(A_full, r, N_nr);
+}
+
+int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr) {
   if (A->n_rows == 0) return 0;
   hipLaunchKernelGGL(k_chunk_reduce, dim3((unsigned)A->n_rows), dim3(256), 0, stream(),
                      A->chunk_base, r, partials, N_nr);
@@ -551,8 +560,9 @@ static int spmm_t_slices(int64_t /*n*/, int r) {
   return 1;
 }
 
-int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
+int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_mr) {
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
+  const dnpeff_csr* A = sparse_part(A_full);
   DN_CHECK(A->colptr != nullptr, "matrix has no transposed copy");
   if (A->n_cols == 0) return 0;
   const bool aligned = ((uintptr_t)T_mr % 16) == 0 && ((uintptr_t)W_nr % 16) == 0;
@@ -594,7 +604,9 @@ int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
     return 0;
   });
   DN_LAUNCH_CHECK();
-  return 0;
+  // the head's rows of the result were stored as zeros above (its columns are empty in the
+  // sparse part); the dense product overwrites them
+  return launch_head_t(A_full, r, W_nr, T_mr);
 }
 
 int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials) {
@@ -628,15 +640,15 @@ using namespace dn;
 DN_API int dnpeff_op_spmm_n(dnpeff_csr* A, int r, const float* H_mr, float* N_nr) {
   clear_error();
   DN_CHECK(A && H_mr && N_nr, "NULL argument");
-  DN_TRY(csr_ensure_partials(A, r));
-  DN_TRY(launch_spmm_n(A, r, H_mr, N_nr, A->partials));
-  return launch_spmm_n_reduce(A, r, A->partials, N_nr);
+  DN_TRY(csr_ensure_products(A, r));
+  DN_TRY(launch_spmm_n(A, r, H_mr));
+  return launch_spmm_n_reduce(A, r, N_nr);
 }
 
 DN_API int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
   clear_error();
   DN_CHECK(A && W_nr && T_mr, "NULL argument");
-  DN_TRY(dnpeff_csr_build_transpose(A));
+  DN_TRY(csr_ensure_products(A, r));
   return launch_spmm_t(A, r, W_nr, T_mr);
 }
 
@@ -646,6 +658,7 @@ DN_API int dnpeff_op_spsp_dense(dnpeff_csr* A, dnpeff_csr* B, float* out_nr) {
   DN_TRY(dnpeff_csr_build_transpose(B));
   const int r = (int)B->n_rows;
   DN_TRY(csr_ensure_partials(A, r));
+  DN_CHECK(!A->tail && !B->tail, "sparse-sparse product of matrices with a dense head");
   DN_TRY(launch_spsp(A, B, A->partials));
-  return launch_spmm_n_reduce(A, r, A->partials, out_nr);
+  return launch_chunk_reduce(A, r, A->partials, out_nr);
 }

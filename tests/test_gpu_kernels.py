@@ -178,3 +178,68 @@ def test_spmm_t_more_columns_than_one_pass_of_the_grid():
     mask[used] = False
     assert not T[mask].any()
     A.close()
+
+
+def _hot_column_matrix(rng, n, m, hot, k_tail, dup=False):
+    """Rows holding most of `hot` columns (each kept with probability 0.8) plus random others."""
+    hot_cols = rng.choice(m, size=hot, replace=False)
+    others = np.setdiff1d(np.arange(m), hot_cols)
+    rowptr, cols, vals = [0], [], []
+    for i in range(n):
+        c = np.concatenate([hot_cols[rng.random(hot) < 0.8],
+                            rng.choice(others, size=int(rng.integers(0, k_tail + 1)), replace=False)])
+        if dup and i % 7 == 0 and len(c):
+            c = np.concatenate([c, c[:3]])  # repeated (row, column) pairs add up
+        rng.shuffle(c)
+        cols.append(c.astype(np.int32))
+        vals.append(rng.lognormal(-2.0, 1.0, size=len(c)).astype(np.float32))
+        rowptr.append(rowptr[-1] + len(c))
+    return (np.array(rowptr, dtype=np.int64), np.concatenate(cols).astype(np.int32),
+            np.concatenate(vals).astype(np.float32), np.sort(hot_cols))
+
+
+@pytest.mark.parametrize("n,m,hot,r", [(300, 4000, 70, 128), (1030, 9000, 300, 64), (257, 3000, 129, 256),
+                                       (140, 2000, 40, 36), (500, 2500, 33, 512)])
+def test_dense_head_products(n, m, hot, r):
+    """Columns held by many rows move to a dense block; A H^T and A^T W stay the same sums."""
+    rng = np.random.default_rng(n + r)
+    rp, ci, va, hot_cols = _hot_column_matrix(rng, n, m, hot, 40, dup=(r == 64))
+    A = d.Csr.from_host(rp, ci, va, m)
+    H = rng.random((m, r)).astype(np.float32)
+    W = rng.random((n, r)).astype(np.float32)
+    dH, dW = d.DeviceArray.from_numpy(H), d.DeviceArray.from_numpy(W)
+    dN, dT = d.DeviceArray((n, r)), d.DeviceArray((m, r))
+    n_dense = A.split_dense_head(0.5)
+    assert n_dense == hot
+    nd, z_sparse = A.head_info()
+    in_head = np.isin(ci, hot_cols)
+    assert nd == hot and z_sparse == int((~in_head).sum())
+    d.op_spmm_n(A, r, dH, dN)
+    d.op_spmm_t(A, r, dW, dT)
+    N, T = dN.numpy(), dT.numpy()
+    N64, T64 = orc.spmm_n_f64(rp, ci, va, H), orc.spmm_t_f64(rp, ci, va, m, W)
+    # row-wise: a wrong head row must not hide behind a large one
+    assert (np.abs(N - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
+    scale = np.maximum(np.abs(T64).max(axis=1), 1e-30)
+    assert (np.abs(T - T64).max(axis=1) / scale)[np.abs(T64).max(axis=1) > 0].max() < TOL
+    assert np.all(T[np.abs(T64).max(axis=1) == 0] == 0)
+    # the loader still sees the whole matrix, and the split can be undone
+    rp2, ci2, va2 = A.download()
+    assert np.array_equal(ci2, ci) and np.array_equal(va2, va)
+    d.op_spmm_n(A, r, dH, dN)
+    assert np.array_equal(dN.numpy(), N)
+    assert A.split_dense_head(0.0) == 0 and A.head_info() == (0, len(ci))
+    d.op_spmm_n(A, r, dH, dN)
+    assert _rel(dN.numpy(), N64) < TOL
+    A.close()
+
+
+def test_dense_head_needs_rank_multiple_of_4():
+    rng = np.random.default_rng(3)
+    rp, ci, va, _ = _hot_column_matrix(rng, 100, 1000, 20, 10)
+    A = d.Csr.from_host(rp, ci, va, 1000)
+    assert A.split_dense_head(0.5) == 20
+    H = d.DeviceArray.from_numpy(rng.random((1000, 50)).astype(np.float32))
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        d.op_spmm_n(A, 50, H, d.DeviceArray((100, 50)))
+    A.close()

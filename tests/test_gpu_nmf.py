@@ -149,3 +149,24 @@ def test_fit_path_first_stage_and_loop():
     lrn.close()
     A.close()
     H.close()
+
+
+def test_dense_head_run_matches_oracle_and_unsplit_run(monkeypatch):
+    """n >= 1024 rows and r >= 64: dnpeff_nmf_create moves the columns most rows hold into the
+    dense block by itself; the run stays within the bar of the fp64 oracle and close to the run
+    with the split switched off."""
+    n, m_full, k, r, eps, iters, seed = 1100, 60000, 3000, 64, 1e-8, 50, 77
+    nmf, A, (W0, H0), (W, H), (W64, H64), hist, losses64 = _run_case(n, m_full, k, r, eps, iters, seed)
+    nd, z_sparse = A.head_info()
+    assert nd > 100 and z_sparse < A.nnz
+    assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
+    got = np.array([h[1] for h in hist])
+    assert np.all(np.abs(got - losses64) / losses64 < REL)
+    nmf.close()
+    A.close()
+    monkeypatch.setenv("DNPEFF_DENSE_FILL", "0")
+    nmf2, A2, _, (W2, H2), _, hist2, _ = _run_case(n, m_full, k, r, eps, iters, seed)
+    assert A2.head_info()[0] == 0
+    assert _nrm(W2, W64) < REL and _nrm(H2, H64) < REL
+    nmf2.close()
+    A2.close()
