@@ -522,6 +522,157 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
+// ---------------------------------------------------------------------------
+// out = X * num / (X G + eps) for r <= 128 (r % 4 == 0): G in registers, X through LDS.
+//
+// With r <= 128 the B operands of a wave -- the 32 columns of G of its column block, all r rows
+// -- fit its registers (r / 2 per lane), so LDS is free for the X tiles: a workgroup streams
+// tiles of ROWS rows through two LDS slots, fetched with coalesced 16-byte loads one tile
+// ahead, and two workgroups share a CU, one running MFMAs while the other is in its epilogue.
+// A wave owns column block cb and two row blocks; lane (i = l%32, half = l/32) reads
+// X[row i][8 kg + 4 half .. + 3] of a row block with one 16-byte LDS read (rows padded by 4
+// floats: conflict free) and MFMA step s contracts component 8 kg + 4 half + s against the
+// matching row of G.  The X factor of the update comes from the same LDS tile.
+// ---------------------------------------------------------------------------
+template <int CB>
+struct XgReg {
+  static constexpr int WPC = 4 / CB;         // waves per column block
+  static constexpr int RB = 2;               // row blocks per wave
+  static constexpr int ROWS = 32 * RB * WPC;  // rows of a tile
+  static constexpr int RP = 32 * CB;          // padded rank
+  static constexpr int LD = RP + 4;
+  static constexpr int KG = RP / 8;
+  static constexpr int C4 = RP / 4;          // 16-byte columns of a tile row
+  static constexpr int RSTEP = 256 / C4;
+  static constexpr int NV = ROWS / RSTEP;    // 16-byte pieces per thread and tile
+  static constexpr int SLOT = ROWS * LD;
+};
+
+template <int CB>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_xg_mu_reg(const float* __restrict__ X, const float* __restrict__ G, const float* num,
+                float eps, int64_t rows, int r, float* out, float* __restrict__ D_out) {
+  using C = XgReg<CB>;
+  extern __shared__ __align__(16) float xl[];  // 2 slots of ROWS x LD
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int cb = wave % CB, rg = wave / CB;
+  const int col = 32 * cb + l32;
+  const bool cok = col < r;
+  const int64_t n_tiles = (rows + C::ROWS - 1) / C::ROWS;
+
+  float g[C::KG][4];
+#pragma unroll
+  for (int kg = 0; kg < C::KG; kg++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int k = 8 * kg + 4 * half + s;
+      g[kg][s] = (k < r && cok) ? G[(int64_t)k * r + col] : 0.0f;
+    }
+
+  const int lc = threadIdx.x % C::C4, lr = threadIdx.x / C::C4;
+  const bool lcok = 4 * lc < r;
+  float4 R[C::NV];
+  auto fetch = [&](int64_t tile) {
+#pragma unroll
+    for (int q = 0; q < C::NV; q++) {
+      const int64_t row = tile * C::ROWS + lr + q * C::RSTEP;
+      const bool ok = lcok && tile < n_tiles && row < rows;
+      R[q] = ok ? *reinterpret_cast<const float4*>(X + row * (int64_t)r + 4 * lc)
+                : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  auto commit = [&](float* slot) {
+#pragma unroll
+    for (int q = 0; q < C::NV; q++)
+      *reinterpret_cast<float4*>(slot + (lr + q * C::RSTEP) * C::LD + 4 * lc) = R[q];
+  };
+
+  int64_t tile = blockIdx.x;
+  fetch(tile);
+  commit(xl);
+  fetch(tile + gridDim.x);
+  __syncthreads();
+
+  for (int it = 0; tile < n_tiles; it++, tile += gridDim.x) {
+    const float* slot = xl + (it & 1) * C::SLOT;
+    const int64_t row0 = tile * C::ROWS + 32 * C::RB * rg;
+    // numerators in the accumulator layout: requested now, they arrive while the MFMAs run
+    float pn[C::RB][16];
+#pragma unroll
+    for (int b = 0; b < C::RB; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int64_t row = row0 + 32 * b + 8 * (v >> 2) + 4 * half + (v & 3);
+        pn[b][v] = (cok && row < rows) ? num[row * (int64_t)r + col] : 0.0f;
+      }
+    acc16 acc[C::RB];
+#pragma unroll
+    for (int b = 0; b < C::RB; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[b][v] = 0.0f;
+
+    const float* arow = slot + (32 * C::RB * rg + l32) * C::LD + 4 * half;
+#pragma unroll
+    for (int kg = 0; kg < C::KG; kg++) {
+      float4 a[C::RB];
+#pragma unroll
+      for (int b = 0; b < C::RB; b++)
+        a[b] = *reinterpret_cast<const float4*>(arow + 32 * b * C::LD + 8 * kg);
+#pragma unroll
+      for (int b = 0; b < C::RB; b++) {
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].x, g[kg][0], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].y, g[kg][1], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].z, g[kg][2], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].w, g[kg][3], acc[b], 0, 0, 0);
+      }
+    }
+
+    if (cok) {
+#pragma unroll
+      for (int b = 0; b < C::RB; b++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int lrow = 32 * C::RB * rg + 32 * b + 8 * (v >> 2) + 4 * half + (v & 3);
+          const int64_t row = tile * C::ROWS + lrow;
+          if (row < rows) {
+            const int64_t idx = row * (int64_t)r + col;
+            const float d = acc[b][v];
+            const float q = pn[b][v] / (d + eps);
+            out[idx] = slot[lrow * C::LD + col] * q;
+            if (D_out) D_out[idx] = d;
+          }
+        }
+    }
+
+    // the other slot was last read before the previous barrier: it takes the next tile, whose
+    // loads were issued one tile ago; the registers then take the tile after it
+    commit(xl + ((it + 1) & 1) * C::SLOT);
+    fetch(tile + 2 * (int64_t)gridDim.x);
+    __syncthreads();
+  }
+}
+
+template <int CB>
+static int launch_xg_mu_reg(int64_t rows, int r, const float* X, const float* G, const float* num,
+                            float eps, float* out, float* D_out) {
+  using C = XgReg<CB>;
+  const size_t lds = sizeof(float) * 2 * C::SLOT;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_reg<CB>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  int64_t tiles = ceil_div(rows, C::ROWS);
+  int64_t wgs = (int64_t)n_cus() * 2;
+  if (wgs > tiles) wgs = tiles;
+  hipLaunchKernelGGL((k_xg_mu_reg<CB>), dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps,
+                     rows, r, out, D_out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
 template <int NB, int PD, bool VEC4>
 static int launch_xg_mu_inst(dim3 grid, size_t lds, const float* X, const float* G,
                              const float* num, float eps, int64_t rows, int r, int nsteps,
@@ -566,6 +717,12 @@ int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const floa
   DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
   DN_CHECK(out != X, "xg_mu: out must not alias X");
   if (rows <= 0) return 0;
+  const bool aligned = ((uintptr_t)X % 16) == 0;
+  if (r % 4 == 0 && r <= 128 && aligned && rows >= 256) {
+    if (r > 64) return launch_xg_mu_reg<4>(rows, r, X, G, num, eps, out, D_out);
+    if (r > 32) return launch_xg_mu_reg<2>(rows, r, X, G, num, eps, out, D_out);
+    return launch_xg_mu_reg<1>(rows, r, X, G, num, eps, out, D_out);
+  }
   // widest column chunk whose slice of G fits 128 KB of LDS
   if (r <= 256) return launch_xg_mu_nb<4>(rows, r, X, G, num, eps, out, D_out);
   if (r <= 512) return launch_xg_mu_nb<2>(rows, r, X, G, num, eps, out, D_out);
