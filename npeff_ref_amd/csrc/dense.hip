@@ -523,7 +523,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 // ---------------------------------------------------------------------------
-// out = X * num / (X G + eps) for r <= 128 (r % 4 == 0): G in registers, X through LDS.
+// out = X * num / (X G + eps) for r = 32, 64 or 128: G in registers, X through LDS.
 //
 // With r <= 128 the B operands of a wave -- the 32 columns of G of its column block, all r rows
 // -- fit its registers (r / 2 per lane), so LDS is free for the X tiles: a workgroup streams
@@ -532,55 +532,52 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 // A wave owns column block cb and two row blocks; lane (i = l%32, half = l/32) reads
 // X[row i][8 kg + 4 half .. + 3] of a row block with one 16-byte LDS read (rows padded by 4
 // floats: conflict free) and MFMA step s contracts component 8 kg + 4 half + s against the
-// matching row of G.  The X factor of the update comes from the same LDS tile.
+// matching row of G.  The X factor of the update comes from the same LDS tile.  The rank is a
+// compile-time constant and the launch covers whole tiles only (the host hands the last rows to
+// k_xg_mu): the epilogue is then straight-line code with one per-lane offset, whose loads, LDS
+// reads and stores the compiler batches; code for partial tiles would cost registers that the
+// main path needs.
 // ---------------------------------------------------------------------------
 template <int CB>
 struct XgReg {
   static constexpr int WPC = 4 / CB;         // waves per column block
   static constexpr int RB = 2;               // row blocks per wave
   static constexpr int ROWS = 32 * RB * WPC;  // rows of a tile
-  static constexpr int RP = 32 * CB;          // padded rank
-  static constexpr int LD = RP + 4;
-  static constexpr int KG = RP / 8;
-  static constexpr int C4 = RP / 4;          // 16-byte columns of a tile row
+  static constexpr int R = 32 * CB;           // rank
+  static constexpr int LD = R + 4;
+  static constexpr int KG = R / 8;
+  static constexpr int C4 = R / 4;           // 16-byte columns of a tile row
   static constexpr int RSTEP = 256 / C4;
   static constexpr int NV = ROWS / RSTEP;    // 16-byte pieces per thread and tile
   static constexpr int SLOT = ROWS * LD;
 };
 
-template <int CB>
+template <int CB, bool WITH_D>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_xg_mu_reg(const float* __restrict__ X, const float* __restrict__ G, const float* num,
-                float eps, int64_t rows, int r, float* out, float* __restrict__ D_out) {
+                float eps, int64_t n_tiles, float* out, float* __restrict__ D_out) {
   using C = XgReg<CB>;
+  constexpr int r = C::R;
   extern __shared__ __align__(16) float xl[];  // 2 slots of ROWS x LD
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int cb = wave % CB, rg = wave / CB;
   const int col = 32 * cb + l32;
-  const bool cok = col < r;
-  const int64_t n_tiles = (rows + C::ROWS - 1) / C::ROWS;
 
   float g[C::KG][4];
 #pragma unroll
   for (int kg = 0; kg < C::KG; kg++)
 #pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const int k = 8 * kg + 4 * half + s;
-      g[kg][s] = (k < r && cok) ? G[(int64_t)k * r + col] : 0.0f;
-    }
+    for (int s = 0; s < 4; s++) g[kg][s] = G[(8 * kg + 4 * half + s) * r + col];
 
   const int lc = threadIdx.x % C::C4, lr = threadIdx.x / C::C4;
-  const bool lcok = 4 * lc < r;
   float4 R[C::NV];
   auto fetch = [&](int64_t tile) {
+    const float* src = X + (tile * C::ROWS + lr) * (int64_t)r + 4 * lc;
 #pragma unroll
-    for (int q = 0; q < C::NV; q++) {
-      const int64_t row = tile * C::ROWS + lr + q * C::RSTEP;
-      const bool ok = lcok && tile < n_tiles && row < rows;
-      R[q] = ok ? *reinterpret_cast<const float4*>(X + row * (int64_t)r + 4 * lc)
-                : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    }
+    for (int q = 0; q < C::NV; q++)
+      R[q] = tile < n_tiles ? *reinterpret_cast<const float4*>(src + q * C::RSTEP * r)
+                            : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   };
   auto commit = [&](float* slot) {
 #pragma unroll
@@ -594,18 +591,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   fetch(tile + gridDim.x);
   __syncthreads();
 
+  // element (b, v) of the accumulators sits 32 b + 8 (v / 4) + v % 4 rows below the lane's
+  // first one: a uniform pointer per row plus one per-lane offset
+  const int lrow0 = 32 * C::RB * rg + 4 * half;
+  const unsigned off0 = (unsigned)(lrow0 * r + col);
+
   for (int it = 0; tile < n_tiles; it++, tile += gridDim.x) {
     const float* slot = xl + (it & 1) * C::SLOT;
-    const int64_t row0 = tile * C::ROWS + 32 * C::RB * rg;
+    const int64_t t0 = tile * C::ROWS * (int64_t)r;
+    const float* tnum = num + t0;
+    float* tout = out + t0;
+    float* tD = WITH_D ? D_out + t0 : nullptr;
     // numerators in the accumulator layout: requested now, they arrive while the MFMAs run
     float pn[C::RB][16];
 #pragma unroll
     for (int b = 0; b < C::RB; b++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int64_t row = row0 + 32 * b + 8 * (v >> 2) + 4 * half + (v & 3);
-        pn[b][v] = (cok && row < rows) ? num[row * (int64_t)r + col] : 0.0f;
-      }
+      for (int v = 0; v < 16; v++)
+        pn[b][v] = (tnum + (32 * b + 8 * (v >> 2) + (v & 3)) * r)[off0];
     acc16 acc[C::RB];
 #pragma unroll
     for (int b = 0; b < C::RB; b++)
@@ -628,21 +631,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
     }
 
-    if (cok) {
 #pragma unroll
-      for (int b = 0; b < C::RB; b++)
+    for (int b = 0; b < C::RB; b++) {
+      float x[16];
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const int lrow = 32 * C::RB * rg + 32 * b + 8 * (v >> 2) + 4 * half + (v & 3);
-          const int64_t row = tile * C::ROWS + lrow;
-          if (row < rows) {
-            const int64_t idx = row * (int64_t)r + col;
-            const float d = acc[b][v];
-            const float q = pn[b][v] / (d + eps);
-            out[idx] = slot[lrow * C::LD + col] * q;
-            if (D_out) D_out[idx] = d;
-          }
-        }
+      for (int v = 0; v < 16; v++)
+        x[v] = slot[(lrow0 + 32 * b + 8 * (v >> 2) + (v & 3)) * C::LD + col];
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int below = (32 * b + 8 * (v >> 2) + (v & 3)) * r;
+        const float d = acc[b][v];
+        const float q = pn[b][v] / (d + eps);
+        (tout + below)[off0] = x[v] * q;
+        if (WITH_D) (tD + below)[off0] = d;
+      }
     }
 
     // the other slot was last read before the previous barrier: it takes the next tile, whose
@@ -653,22 +655,31 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
+// rows must be a multiple of XgReg<CB>::ROWS
 template <int CB>
-static int launch_xg_mu_reg(int64_t rows, int r, const float* X, const float* G, const float* num,
+static int launch_xg_mu_reg(int64_t rows, const float* X, const float* G, const float* num,
                             float eps, float* out, float* D_out) {
   using C = XgReg<CB>;
   const size_t lds = sizeof(float) * 2 * C::SLOT;
   static bool attr_set = false;
   if (!attr_set) {
-    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_reg<CB>,
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_reg<CB, false>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_reg<CB, true>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
-  int64_t tiles = ceil_div(rows, C::ROWS);
+  const int64_t tiles = rows / C::ROWS;
+  if (tiles == 0) return 0;
   int64_t wgs = (int64_t)n_cus() * 2;
   if (wgs > tiles) wgs = tiles;
-  hipLaunchKernelGGL((k_xg_mu_reg<CB>), dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps,
-                     rows, r, out, D_out);
+  const dim3 grid((unsigned)wgs), block(256);
+  if (D_out)
+    hipLaunchKernelGGL((k_xg_mu_reg<CB, true>), grid, block, lds, stream(), X, G, num, eps, tiles,
+                       out, D_out);
+  else
+    hipLaunchKernelGGL((k_xg_mu_reg<CB, false>), grid, block, lds, stream(), X, G, num, eps, tiles,
+                       out, D_out);
   DN_LAUNCH_CHECK();
   return 0;
 }
@@ -718,10 +729,23 @@ int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const floa
   DN_CHECK(out != X, "xg_mu: out must not alias X");
   if (rows <= 0) return 0;
   const bool aligned = ((uintptr_t)X % 16) == 0;
-  if (r % 4 == 0 && r <= 128 && aligned && rows >= 256) {
-    if (r > 64) return launch_xg_mu_reg<4>(rows, r, X, G, num, eps, out, D_out);
-    if (r > 32) return launch_xg_mu_reg<2>(rows, r, X, G, num, eps, out, D_out);
-    return launch_xg_mu_reg<1>(rows, r, X, G, num, eps, out, D_out);
+  if ((r == 32 || r == 64 || r == 128) && aligned && rows >= 256) {
+    // whole tiles with the compile-time-rank kernel, the last rows below
+    int64_t head;
+    if (r == 128) {
+      head = rows / XgReg<4>::ROWS * XgReg<4>::ROWS;
+      DN_TRY(launch_xg_mu_reg<4>(head, X, G, num, eps, out, D_out));
+    } else if (r == 64) {
+      head = rows / XgReg<2>::ROWS * XgReg<2>::ROWS;
+      DN_TRY(launch_xg_mu_reg<2>(head, X, G, num, eps, out, D_out));
+    } else {
+      head = rows / XgReg<1>::ROWS * XgReg<1>::ROWS;
+      DN_TRY(launch_xg_mu_reg<1>(head, X, G, num, eps, out, D_out));
+    }
+    if (head == rows) return 0;
+    const int64_t off = head * r;
+    return launch_xg_mu_nb<4>(rows - head, r, X + off, G, num + off, eps, out + off,
+                              D_out ? D_out + off : nullptr);
   }
   // widest column chunk whose slice of G fits 128 KB of LDS
   if (r <= 256) return launch_xg_mu_nb<4>(rows, r, X, G, num, eps, out, D_out);
