@@ -144,6 +144,13 @@ struct dnpeff_csr {
   // workspace for the per-chunk partial sums of A H^T ([n_chunks, r])
   float* partials = nullptr;
   int64_t partials_floats = 0;
+  // column panels of A H^T: the entries of every row regrouped by panel (original order kept
+  // inside a panel), seg[row * (n_panels + 1) + p] = first entry of the (row, p) segment
+  int n_panels = 0;
+  int32_t* panel_bounds = nullptr;  // [n_panels + 1] first column of each panel
+  int64_t* seg = nullptr;
+  int32_t* pcol = nullptr;
+  float* pval = nullptr;
   // after dnpeff_csr_split_dense_head: the dense block and the matrix of the remaining entries
   // (same shape, owned), which carries the derived structures the products use
   dn::dense_head head;
@@ -155,6 +162,9 @@ inline dnpeff_csr* sparse_part(dnpeff_csr* A) { return A->tail ? A->tail : A; }
 inline const dnpeff_csr* sparse_part(const dnpeff_csr* A) { return A->tail ? A->tail : A; }
 int csr_ensure_chunks(dnpeff_csr* A);
 int csr_ensure_partials(dnpeff_csr* A, int r);
+// Builds (or drops) the column panels of a matrix without dense head / of a sparse part;
+// needs the transposed copy.  n_panels = 0 removes them.
+int csr_set_panels(dnpeff_csr* S, int n_panels);
 // Everything A H^T and A^T W at rank r need: transposed copy and work lists of the sparse part,
 // workspaces of the sparse part and of the dense head.
 int csr_ensure_products(dnpeff_csr* A, int r);

@@ -4,6 +4,7 @@
 #include "dnpeff_internal.hpp"
 
 #include <cmath>
+#include <cstdlib>
 
 #include <cstdarg>
 #include <cstring>
@@ -256,6 +257,109 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// bounds[p] = first column c with colptr[c] >= p * nnz / P  (bounds[0] = 0, bounds[P] = n_cols):
+// P panels of consecutive columns with about the same number of entries each.
+__global__ void __launch_bounds__(256)
+    k_panel_bounds(const int64_t* __restrict__ colptr, int64_t n_cols, int64_t nnz, int P,
+                   int32_t* __restrict__ bounds) {
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  if (p > P) return;
+  if (p == 0) { bounds[0] = 0; return; }
+  if (p == P) { bounds[P] = (int32_t)n_cols; return; }
+  const int64_t target = (int64_t)(((__int128)nnz * p) / P);
+  int64_t lo = 0, hi = n_cols;  // smallest c in [0, n_cols] with colptr[c] >= target
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (colptr[mid] >= target) hi = mid; else lo = mid + 1;
+  }
+  bounds[p] = (int32_t)lo;
+}
+
+// Regroups the entries of each row by column panel, keeping their order inside a panel (a
+// stable split, so the result does not depend on how the hardware schedules the lanes), and
+// records where each (row, panel) segment starts.  One workgroup per row at a time: a counting
+// pass, a scan over the panels, then tiles of 256 entries in order; within a tile an entry's
+// rank among the entries of its panel comes from wave ballots over the bits of the panel
+// number plus the per-wave counts of the earlier waves.
+constexpr int MAX_PANELS = 256;
+
+__global__ void __launch_bounds__(256)
+    k_panel_split(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
+                  const float* __restrict__ vals, int64_t n_rows, int P, int bits,
+                  const int32_t* __restrict__ bounds, int64_t* __restrict__ seg,
+                  int32_t* __restrict__ pcol, float* __restrict__ pval) {
+  __shared__ int32_t bnd[MAX_PANELS + 1];
+  __shared__ int hist[MAX_PANELS];
+  __shared__ int64_t cursor[MAX_PANELS];
+  __shared__ int wcnt[4][MAX_PANELS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  for (int i = tid; i <= P; i += 256) bnd[i] = bounds[i];
+  auto panel_of = [&](int32_t col) {
+    int lo = 0, hi = P;  // largest p < P with bnd[p] <= col
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (bnd[mid] <= col) lo = mid; else hi = mid;
+    }
+    return lo;
+  };
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    const int64_t e0 = rowptr[row], e1 = rowptr[row + 1];
+    __syncthreads();
+    for (int i = tid; i < P; i += 256) {
+      hist[i] = 0;
+      wcnt[0][i] = wcnt[1][i] = wcnt[2][i] = wcnt[3][i] = 0;
+    }
+    __syncthreads();
+    for (int64_t e = e0 + tid; e < e1; e += 256) atomicAdd(&hist[panel_of(colind[e])], 1);
+    __syncthreads();
+    for (int i = tid; i < P; i += 256) {
+      int64_t s = 0;
+      for (int q = 0; q < i; q++) s += hist[q];
+      cursor[i] = e0 + s;
+      seg[row * (P + 1) + i] = e0 + s;
+    }
+    if (tid == 0) seg[row * (P + 1) + P] = e1;
+    __syncthreads();
+    for (int64_t base = e0; base < e1; base += 256) {
+      const int64_t e = base + tid;
+      const bool active = e < e1;
+      int32_t col = 0;
+      float v = 0.0f;
+      int pid = 0;
+      if (active) {
+        col = colind[e];
+        v = vals[e];
+        pid = panel_of(col);
+      }
+      unsigned long long mask = __ballot(active);
+      for (int b = 0; b < bits; b++) {
+        const bool bit = (pid >> b) & 1;
+        const unsigned long long bal = __ballot(active && bit);
+        mask &= bit ? bal : ~bal;
+      }
+      const int rank = __popcll(mask & ((1ull << lane) - 1ull));
+      if (active && rank == 0) wcnt[wave][pid] = __popcll(mask);
+      __syncthreads();
+      if (active) {
+        int off = 0;
+        for (int w = 0; w < wave; w++) off += wcnt[w][pid];
+        const int64_t pos = cursor[pid] + off + rank;
+        pcol[pos] = col;
+        pval[pos] = v;
+      }
+      __syncthreads();
+      for (int i = tid; i < P; i += 256) {
+        const int tot = wcnt[0][i] + wcnt[1][i] + wcnt[2][i] + wcnt[3][i];
+        if (tot) {
+          cursor[i] += tot;
+          wcnt[0][i] = wcnt[1][i] = wcnt[2][i] = wcnt[3][i] = 0;
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
 __global__ void __launch_bounds__(256) k_fill_i32(int32_t* p, int64_t n, int32_t v) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) p[i] = v;
@@ -397,8 +501,20 @@ static void drop_head(dnpeff_csr* A) {
   A->head = dense_head();
 }
 
+static void drop_panels(dnpeff_csr* A) {
+  dfree(A->panel_bounds); A->panel_bounds = nullptr;
+  dfree(A->seg); A->seg = nullptr;
+  dfree(A->pcol); A->pcol = nullptr;
+  dfree(A->pval); A->pval = nullptr;
+  if (A->n_panels) {  // the partial sums were sized for the panels
+    dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
+  }
+  A->n_panels = 0;
+}
+
 static void drop_derived(dnpeff_csr* A) {
   drop_head(A);
+  drop_panels(A);
   dfree(A->colptr); A->colptr = nullptr;
   dfree(A->rowind); A->rowind = nullptr;
   dfree(A->tvals); A->tvals = nullptr;
@@ -417,9 +533,58 @@ int csr_ensure_chunks(dnpeff_csr* A) {
   return 0;
 }
 
+int csr_set_panels(dnpeff_csr* S, int P) {
+  if (P == S->n_panels) return 0;
+  drop_panels(S);
+  if (P <= 0) return 0;
+  DN_CHECK(P <= MAX_PANELS, "at most %d column panels", MAX_PANELS);
+  DN_CHECK(S->rowptr && S->colptr, "column panels need both copies of the matrix");
+  hipStream_t st = stream();
+  int bits = 0;
+  while ((1 << bits) < P) bits++;
+  int s = dmalloc(&S->panel_bounds, (int64_t)P + 1) || dmalloc(&S->seg, S->n_rows * (P + 1)) ||
+          dmalloc(&S->pcol, S->nnz) || dmalloc(&S->pval, S->nnz);
+  if (!s) {
+    hipLaunchKernelGGL(k_panel_bounds, dim3((unsigned)ceil_div(P + 1, 256)), dim3(256), 0, st,
+                       S->colptr, S->n_cols, S->nnz, P, S->panel_bounds);
+    int64_t wgs = S->n_rows < 8192 ? S->n_rows : 8192;
+    hipLaunchKernelGGL(k_panel_split, dim3((unsigned)(wgs < 1 ? 1 : wgs)), dim3(256), 0, st, S->rowptr,
+                       S->colind, S->vals, S->n_rows, P, bits, S->panel_bounds, S->seg, S->pcol,
+                       S->pval);
+    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(st) != hipSuccess) {
+      set_error("building the column panels failed");
+      s = 1;
+    }
+  }
+  if (s) { drop_panels(S); return s; }
+  S->n_panels = P;
+  dfree(S->partials); S->partials = nullptr; S->partials_floats = 0;
+  return 0;
+}
+
+// Panels pay when the gathered factor [n_cols, r] is far larger than the caches and there are
+// rows enough to share a panel's part of it: one panel per ~96 MB of the factor, 8..256, and
+// few enough for the (panel, 4 rows) workgroups to fit one launch.  DNPEFF_PANELS overrides the
+// number (0 = none).
+static int panel_policy(const dnpeff_csr* S, int r) {
+  int64_t P = 0;
+  const double bytes = 4.0 * (double)S->n_cols * r;
+  if (bytes >= 512e6 && S->n_rows >= 64) {
+    P = (int64_t)ceil(bytes / 96e6);
+    if (P < 8) P = 8;
+  }
+  if (const char* e = getenv("DNPEFF_PANELS")) P = atoi(e);
+  if (P > MAX_PANELS) P = MAX_PANELS;
+  const int64_t row_groups = ceil_div(S->n_rows, 4);
+  while (P > 1 && P * row_groups >= ((int64_t)1 << 24)) P /= 2;
+  if (P < 2 || S->nnz == 0) P = 0;
+  return (int)P;
+}
+
 int csr_ensure_products(dnpeff_csr* A, int r) {
   dnpeff_csr* S = sparse_part(A);
   DN_TRY(dnpeff_csr_build_transpose(S));
+  DN_TRY(csr_set_panels(S, panel_policy(S, r)));
   DN_TRY(csr_ensure_partials(S, r));
   return head_ensure_workspace(A, r);
 }
@@ -427,6 +592,8 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
 int csr_ensure_partials(dnpeff_csr* A, int r) {
   DN_TRY(csr_ensure_chunks(A));
   int64_t need = A->n_chunks * (int64_t)r;
+  if (A->n_panels > 0 && A->n_rows * A->n_panels * (int64_t)r > need)
+    need = A->n_rows * A->n_panels * (int64_t)r;
   if (need <= A->partials_floats && A->partials) return 0;
   dfree(A->partials);
   A->partials = nullptr;

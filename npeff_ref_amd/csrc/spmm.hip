@@ -219,6 +219,46 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---------------------------------------------------------------------------
+// Column panels.  When H is far larger than the caches, every gathered row of H comes from
+// HBM unless the workgroups running at one time gather from the same part of H.  The entries of
+// each row are therefore regrouped by column panel (same panels for all rows, equal numbers of
+// entries per panel over the whole matrix), a wave owns one (row, panel) segment and the grid
+// runs panel by panel: the rows of H of a panel are fetched from HBM once and then found in
+// L2 / the memory-side cache by the other rows' segments.
+// part[row, panel, :] = sum over the segment's entries of val * H[col, :]
+// ---------------------------------------------------------------------------
+template <class GT>
+__global__ void __launch_bounds__(256)
+    k_spmm_n_panel(const int64_t* __restrict__ seg, const int32_t* __restrict__ pcol,
+                   const float* __restrict__ pval, int64_t n_rows, int64_t row_groups, int P, int r,
+                   const float* __restrict__ H, float* __restrict__ part) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int64_t p = blockIdx.x / row_groups;
+  const int64_t row = (blockIdx.x % row_groups) * 4 + wave;
+  if (row >= n_rows) return;
+  const int64_t* sg = seg + row * (P + 1) + p;
+  GT g;
+  g.init(lane, r);
+  g.run(pcol, pval, sg[0], sg[1], H, r);
+  g.store(part + (row * P + p) * r);
+}
+
+// N[row, :] = sum of the row's panel partials, in panel order, accumulated in fp64.
+__global__ void __launch_bounds__(256)
+    k_panel_reduce(const float* __restrict__ part, int64_t n_rows, int P, int r,
+                   float* __restrict__ N) {
+  const int64_t total = n_rows * r, stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int64_t row = e / r;
+    const int c = (int)(e % r);
+    const float* src = part + row * P * r + c;
+    double s = 0.0;
+    for (int p = 0; p < P; p++) s += (double)src[(int64_t)p * r];
+    N[e] = (float)s;
+  }
+}
+
 // N[row, :] = sum of the row's chunk partials, in chunk order.
 __global__ void __launch_bounds__(256)
     k_chunk_reduce(const int64_t* __restrict__ chunk_base, int r,
@@ -519,6 +559,19 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
   DN_TRY(launch_head_n(A_full, r, H_mr));
   const dnpeff_csr* A = sparse_part(A_full);
   float* partials = A->partials;
+  if (A->n_panels > 0) {
+    DN_CHECK(A->seg && A->pcol && partials, "matrix has no panel work list");
+    const int64_t row_groups = ceil_div(A->n_rows, 4);
+    dim3 grid((unsigned)(row_groups * A->n_panels)), block(256);
+    dispatch_gather(r, ((uintptr_t)H_mr % 16) == 0, [&](auto tag) {
+      using GT = typename decltype(tag)::type;
+      hipLaunchKernelGGL((k_spmm_n_panel<GT>), grid, block, 0, stream(), A->seg, A->pcol, A->pval,
+                         A->n_rows, row_groups, A->n_panels, r, H_mr, partials);
+      return 0;
+    });
+    DN_LAUNCH_CHECK();
+    return 0;
+  }
   DN_CHECK(A->rowptr && A->chunk_base && partials, "matrix has no row-major copy / work list");
   if (A->n_chunks == 0) return 0;
   DN_CHECK(A->n_chunks < (int64_t)INT32_MAX, "too many work chunks");
@@ -536,7 +589,17 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
 
 int launch_spmm_n_reduce(const dnpeff_csr* A_full, int r, float* N_nr) {
   const dnpeff_csr* A = sparse_part(A_full);
-  DN_TRY(launch_chunk_reduce(A, r, A->partials, N_nr));
+  if (A->n_panels > 0) {
+    if (A->n_rows > 0) {
+      int64_t wgs = ceil_div(A->n_rows * r, 256);
+      if (wgs > (1 << 20)) wgs = 1 << 20;
+      hipLaunchKernelGGL(k_panel_reduce, dim3((unsigned)wgs), dim3(256), 0, stream(), A->partials,
+                         A->n_rows, A->n_panels, r, N_nr);
+      DN_LAUNCH_CHECK();
+    }
+  } else {
+    DN_TRY(launch_chunk_reduce(A, r, A->partials, N_nr));
+  }
   return launch_head_n_add(A_full, r, N_nr);
 }
 

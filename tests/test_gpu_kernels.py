@@ -245,3 +245,49 @@ def test_dense_head_needs_rank_multiple_of_4():
     with pytest.raises(RuntimeError, match="multiple of 4"):
         d.op_spmm_n(A, 50, H, d.DeviceArray((100, 50)))
     A.close()
+
+
+@pytest.mark.parametrize("panels,r,n,m,maxk", [(8, 128, 130, 5000, 3000), (37, 64, 61, 900, 400), (256, 50, 300, 20000, 700),
+                                               (2, 16, 5, 40, 30)])
+def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
+    """Entries regrouped by column panel, one wave per (row, panel) segment: same sums, same bits
+    on every run, empty rows and empty segments included."""
+    monkeypatch.setenv("DNPEFF_PANELS", str(panels))
+    rng = np.random.default_rng(panels + r)
+    rp, ci, va = random_csr(rng, n, m, maxk, empty_rows={1, n - 1})
+    A = d.Csr.from_host(rp, ci, va, m)
+    H = rng.random((m, r)).astype(np.float32)
+    dH, dN = d.DeviceArray.from_numpy(H), d.DeviceArray((n, r))
+    d.op_spmm_n(A, r, dH, dN)
+    N = dN.numpy()
+    N64 = orc.spmm_n_f64(rp, ci, va, H)
+    assert (np.abs(N - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
+    assert np.all(N[1] == 0) and np.all(N[n - 1] == 0)
+    d.op_spmm_n(A, r, dH, dN)
+    assert np.array_equal(dN.numpy(), N)
+    # the other product and the loader are untouched by the regrouping
+    W = rng.random((n, r)).astype(np.float32)
+    dT = d.DeviceArray((m, r))
+    d.op_spmm_t(A, r, d.DeviceArray.from_numpy(W), dT)
+    assert _rel(dT.numpy(), orc.spmm_t_f64(rp, ci, va, m, W)) < TOL
+    assert np.array_equal(A.download()[1], ci)
+    # without panels: the chunked path again
+    monkeypatch.setenv("DNPEFF_PANELS", "0")
+    d.op_spmm_n(A, r, dH, dN)
+    assert _rel(dN.numpy(), N64) < TOL
+    A.close()
+
+
+def test_column_panels_with_dense_head(monkeypatch):
+    monkeypatch.setenv("DNPEFF_PANELS", "16")
+    rng = np.random.default_rng(11)
+    n, m, r = 400, 6000, 128
+    rp, ci, va, hot_cols = _hot_column_matrix(rng, n, m, 50, 200)
+    A = d.Csr.from_host(rp, ci, va, m)
+    assert A.split_dense_head(0.5) == 50
+    H = rng.random((m, r)).astype(np.float32)
+    dN = d.DeviceArray((n, r))
+    d.op_spmm_n(A, r, d.DeviceArray.from_numpy(H), dN)
+    N64 = orc.spmm_n_f64(rp, ci, va, H)
+    assert (np.abs(dN.numpy() - N64).max(axis=1) / np.abs(N64).max(axis=1)).max() < TOL
+    A.close()

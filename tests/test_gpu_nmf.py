@@ -170,3 +170,13 @@ def test_dense_head_run_matches_oracle_and_unsplit_run(monkeypatch):
     assert _nrm(W2, W64) < REL and _nrm(H2, H64) < REL
     nmf2.close()
     A2.close()
+
+
+def test_column_panel_run_matches_oracle(monkeypatch):
+    monkeypatch.setenv("DNPEFF_PANELS", "12")
+    nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(300, 40000, 2048, 128, 1e-8, 50, seed=5)
+    assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
+    got = np.array([h[1] for h in hist])
+    assert np.all(np.abs(got - losses64) / losses64 < REL)
+    nmf.close()
+    A.close()
