@@ -281,7 +281,7 @@ __global__ void __launch_bounds__(256)
 // pass, a scan over the panels, then tiles of 256 entries in order; within a tile an entry's
 // rank among the entries of its panel comes from wave ballots over the bits of the panel
 // number plus the per-wave counts of the earlier waves.
-constexpr int MAX_PANELS = 256;
+constexpr int MAX_PANELS = 512;
 
 __global__ void __launch_bounds__(256)
     k_panel_split(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
@@ -563,14 +563,16 @@ int csr_set_panels(dnpeff_csr* S, int P) {
 }
 
 // Panels pay when the gathered factor [n_cols, r] is far larger than the caches and there are
-// rows enough to share a panel's part of it: one panel per ~96 MB of the factor, 8..256, and
-// few enough for the (panel, 4 rows) workgroups to fit one launch.  DNPEFF_PANELS overrides the
-// number (0 = none).
+// rows enough to share a panel's part of it: one panel per ~48 MB of the factor, 8..512, and
+// few enough for the (panel, 4 rows) workgroups to fit one launch.  On 10,000 x 65.9M, r = 128
+// (33.7 GB factor): no panels 29.3 ms, 32: 27.8, 128: 23.9, 256: 21.8, 512: 20.1 ms for the
+// gathers, plus 0.1 to 0.8 ms for the sum over panels; 1024 gains 1.1 ms and loses 0.7.
+// DNPEFF_PANELS overrides the number (0 = none).
 static int panel_policy(const dnpeff_csr* S, int r) {
   int64_t P = 0;
   const double bytes = 4.0 * (double)S->n_cols * r;
   if (bytes >= 512e6 && S->n_rows >= 64) {
-    P = (int64_t)ceil(bytes / 96e6);
+    P = (int64_t)ceil(bytes / 48e6);
     if (P < 8) P = 8;
   }
   if (const char* e = getenv("DNPEFF_PANELS")) P = atoi(e);

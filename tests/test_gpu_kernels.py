@@ -247,7 +247,7 @@ def test_dense_head_needs_rank_multiple_of_4():
     A.close()
 
 
-@pytest.mark.parametrize("panels,r,n,m,maxk", [(8, 128, 130, 5000, 3000), (37, 64, 61, 900, 400), (256, 50, 300, 20000, 700),
+@pytest.mark.parametrize("panels,r,n,m,maxk", [(8, 128, 130, 5000, 3000), (37, 64, 61, 900, 400), (256, 50, 300, 20000, 700), (512, 32, 40, 30000, 2000),
                                                (2, 16, 5, 40, 30)])
 def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
     """Entries regrouped by column panel, one wave per (row, panel) segment: same sums, same bits
