@@ -32,6 +32,18 @@ CONFIGS = {
 }
 
 
+# HBM-side bytes per launch of the long kernel of each class on configs[1], from rocprofv3 --pmc
+# FETCH_SIZE (x 2.0) + WRITE_SIZE (x 1.0), the factors being what the same counters read for a
+# plain copy of known size; counters cannot be read from inside this process, so the figures of
+# the committed profile are carried here and apply to the unchanged c1 workload only.
+TRAFFIC_C1 = {
+    "spmm_n": 121.6e9 + 2.6e9,    # sparse part; the dense head adds about 5 GB
+    "spmm_t": 65.5e9 + 33.7e9 + 7.4e9 + 0.1e9,
+    "gram_H": 33.8e9 + 0.1e9,
+    "xg_mu_H": 67.5e9 + 33.8e9,
+}
+
+
 def log(msg):
     print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
 
@@ -172,7 +184,8 @@ def main():
     kd = kernels[dom]
     roofline = dict(kernel=dom, bound=kd["bound"], achieved=kd["achieved"],
                     peak=HBM_PEAK / 1e9 if kd["bound"] == "hbm" else MFMA_FP32_PEAK / 1e12,
-                    unit=kd["unit"], frac=kd["frac"], traffic=None)
+                    unit=kd["unit"], frac=kd["frac"],
+                    traffic=TRAFFIC_C1.get(dom) if args.config == "c1" else None)
 
     cpu_baseline = run_cpu_baseline(cpu, args.cpu_steps, n, m, z, r) if cpu is not None else None
 
