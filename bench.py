@@ -29,6 +29,9 @@ CONFIGS = {
     "c0": dict(n=512, m_full=1 << 20, k=4096, kmin=0, kmax=0, s=1.1, r=16),
     "c1": dict(n=10_000, m_full=110_000_000, k=65_536, kmin=0, kmax=0, s=1.1, r=128),
     "c1-small": dict(n=1_000, m_full=11_000_000, k=16_384, kmin=0, kmax=0, s=1.1, r=128),
+    # downscaled shapes of configs[3] (Zipf 1.3, r = 256) and configs[4] (ragged rows, r = 512)
+    "c3-small": dict(n=5_000, m_full=90_000_000, k=65_536, kmin=0, kmax=0, s=1.3, r=256),
+    "c4-small": dict(n=5_000, m_full=40_000_000, k=0, kmin=1_024, kmax=131_072, s=1.1, r=512),
 }
 
 

@@ -684,6 +684,174 @@ static int launch_xg_mu_reg(int64_t rows, const float* X, const float* G, const 
   return 0;
 }
 
+// ---------------------------------------------------------------------------
+// out = X * num / (X G + eps) for r a multiple of 128 above 128: both operands through LDS.
+//
+// A workgroup owns a 128 x 128 tile of X G (row tile, column chunk) and walks the r components
+// in tiles of 32: the X part [128 rows][32 k] (rows padded to 36 floats: one conflict-free
+// 16-byte LDS read gives a lane 4 consecutive components of its row) and the G part
+// [32 k][128 columns] of the two LDS slots are fetched with coalesced 16-byte loads one tile
+// ahead into registers and committed after the MFMAs of the current tile.  Wave (wm, wn) owns
+// 64 rows x 64 columns (2 x 2 blocks of 32 x 32).  Workgroups of one row tile are neighbours in
+// the grid, so the chunks after the first find the X tile in L2 / the memory-side cache.  The
+// epilogue walks the four blocks with the operands of the next block in flight.
+// ---------------------------------------------------------------------------
+constexpr int XGT_KB = 32;
+constexpr int XGT_XLD = XGT_KB + 4;
+constexpr int XGT_XPART = 128 * XGT_XLD;        // floats
+constexpr int XGT_SLOT = XGT_XPART + XGT_KB * 128;
+
+template <bool WITH_D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_xg_mu_tile(const float* __restrict__ X, const float* __restrict__ G, const float* num,
+                 float eps, int64_t rows, int r, int n_chunks, float* out,
+                 float* __restrict__ D_out) {
+  extern __shared__ __align__(16) float tl[];  // 2 slots
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t tile = blockIdx.x / n_chunks;
+  const int n0 = (int)(blockIdx.x % n_chunks) * 128;
+  const int64_t row0 = tile * 128;
+  const int n_kt = r / XGT_KB;
+
+  // loader roles: X: 16-byte column xc of rows xr + 32 q; G: 16-byte column gc of k gk + 8 q
+  const int xc = threadIdx.x & 7, xr = threadIdx.x >> 3;
+  const int gc = threadIdx.x & 31, gk = threadIdx.x >> 5;
+  float4 RX[4], RG[4];
+  auto fetch = [&](int kt) {
+    const int k0 = kt * XGT_KB;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int64_t row = row0 + xr + 32 * q;
+      RX[q] = (kt < n_kt && row < rows)
+                  ? *reinterpret_cast<const float4*>(X + row * (int64_t)r + k0 + 4 * xc)
+                  : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      RG[q] = kt < n_kt ? *reinterpret_cast<const float4*>(G + (int64_t)(k0 + gk + 8 * q) * r + n0 + 4 * gc)
+                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  auto commit = [&](float* slot) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      *reinterpret_cast<float4*>(slot + (xr + 32 * q) * XGT_XLD + 4 * xc) = RX[q];
+      *reinterpret_cast<float4*>(slot + XGT_XPART + (gk + 8 * q) * 128 + 4 * gc) = RG[q];
+    }
+  };
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+  fetch(0);
+  commit(tl);
+  fetch(1);
+  __syncthreads();
+  for (int kt = 0; kt < n_kt; kt++) {
+    const float* slot = tl + (kt & 1) * XGT_SLOT;
+    const float* pa = slot + (64 * wm + l32) * XGT_XLD + 4 * half;
+    const float* pb = slot + XGT_XPART + 4 * half * 128 + 64 * wn + l32;
+#pragma unroll
+    for (int kg = 0; kg < XGT_KB / 8; kg++) {
+      float4 a[2];
+      float b[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        a[i] = *reinterpret_cast<const float4*>(pa + 32 * i * XGT_XLD + 8 * kg);
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int s2 = 0; s2 < 4; s2++) b[j][s2] = pb[(8 * kg + s2) * 128 + 32 * j];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, b[j][0], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, b[j][1], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, b[j][2], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, b[j][3], acc[i][j], 0, 0, 0);
+        }
+    }
+    // the other slot was last read before the previous barrier
+    commit(tl + ((kt + 1) & 1) * XGT_SLOT);
+    fetch(kt + 2);
+    __syncthreads();
+  }
+
+  // element (i, j, v): row 64 wm + 32 i + 8 (v / 4) + 4 half + v % 4, column n0 + 64 wn + 32 j + l32
+  const int64_t t0 = (row0 + 64 * wm + 4 * half) * (int64_t)r + n0 + 64 * wn;
+  const float* tnum = num + t0;
+  const float* tx = X + t0;
+  float* tout = out + t0;
+  float* tD = WITH_D ? D_out + t0 : nullptr;
+  const int64_t rows_left = rows - (row0 + 64 * wm + 4 * half);  // rows at and below the lane's first
+  float pn[2][16], px[2][16];
+  auto request = [&](int blk, float (&n_)[16], float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int below = 32 * i + 8 * (v >> 2) + (v & 3);
+      // rows past the end are clamped to the lane's first row (never stored)
+      const int64_t off = (below < rows_left ? below : 0) * (int64_t)r + 32 * j + l32;
+      n_[v] = tnum[off];
+      x_[v] = tx[off];
+    }
+  };
+  auto finish = [&](int blk, const float (&n_)[16], const float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int below = 32 * i + 8 * (v >> 2) + (v & 3);
+      if (below < rows_left) {
+        const int64_t off = below * (int64_t)r + 32 * j + l32;
+        const float d = acc[i][j][v];
+        const float q = n_[v] / (d + eps);
+        tout[off] = x_[v] * q;
+        if (WITH_D) tD[off] = d;
+      }
+    }
+  };
+  if (rows_left > 0) {
+    request(0, pn[0], px[0]);
+    request(1, pn[1], px[1]);
+    finish(0, pn[0], px[0]);
+    request(2, pn[0], px[0]);
+    finish(1, pn[1], px[1]);
+    request(3, pn[1], px[1]);
+    finish(2, pn[0], px[0]);
+    finish(3, pn[1], px[1]);
+  }
+}
+
+static int launch_xg_mu_tile(int64_t rows, int r, const float* X, const float* G, const float* num,
+                             float eps, float* out, float* D_out) {
+  const size_t lds = sizeof(float) * 2 * XGT_SLOT;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_tile<false>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_tile<true>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int n_chunks = r / 128;
+  const int64_t wgs = ceil_div(rows, 128) * n_chunks;
+  DN_CHECK(wgs < ((int64_t)1 << 24), "xg_mu: too many tiles for one launch");
+  const dim3 grid((unsigned)wgs), block(256);
+  if (D_out)
+    hipLaunchKernelGGL((k_xg_mu_tile<true>), grid, block, lds, stream(), X, G, num, eps, rows, r,
+                       n_chunks, out, D_out);
+  else
+    hipLaunchKernelGGL((k_xg_mu_tile<false>), grid, block, lds, stream(), X, G, num, eps, rows, r,
+                       n_chunks, out, D_out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
 template <int NB, int PD, bool VEC4>
 static int launch_xg_mu_inst(dim3 grid, size_t lds, const float* X, const float* G,
                              const float* num, float eps, int64_t rows, int r, int nsteps,
@@ -747,6 +915,9 @@ int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const floa
     return launch_xg_mu_nb<4>(rows - head, r, X + off, G, num + off, eps, out + off,
                               D_out ? D_out + off : nullptr);
   }
+  if (r > 128 && r % 128 == 0 && aligned && ((uintptr_t)G % 16) == 0 && rows >= 256 &&
+      ceil_div(rows, 128) * (r / 128) < ((int64_t)1 << 24))
+    return launch_xg_mu_tile(rows, r, X, G, num, eps, out, D_out);
   // widest column chunk whose slice of G fits 128 KB of LDS
   if (r <= 256) return launch_xg_mu_nb<4>(rows, r, X, G, num, eps, out, D_out);
   if (r <= 512) return launch_xg_mu_nb<2>(rows, r, X, G, num, eps, out, D_out);

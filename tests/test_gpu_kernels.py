@@ -85,7 +85,7 @@ def test_gram(rows, r):
 
 @pytest.mark.parametrize("rows,r", [(1, 16), (33, 16), (1000, 50), (4100, 128), (5000, 256), (3000, 512), (300, 130),
                                     (700, 64), (1000, 100), (513, 36), (300, 20), (257, 32), (70001, 128),
-                                    (140000, 64), (256, 128), (255, 128)])
+                                    (140000, 64), (256, 128), (255, 128), (1001, 384), (40000, 256), (257, 1024)])
 def test_xg_mu(rows, r):
     rng = np.random.default_rng(rows * 3 + r)
     X = rng.random((rows, r)).astype(np.float32)
