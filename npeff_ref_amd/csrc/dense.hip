@@ -68,7 +68,10 @@ static int gram_pairs(int r) {
   return nb * (nb + 1) / 2;
 }
 
+static bool gram_uses_tiles(int64_t rows, int r) { return r > 128 && r % 128 == 0 && rows >= 1024; }
+
 int64_t gram_workspace_floats(int64_t rows, int r) {
+  if (gram_uses_tiles(rows, r)) return gram_tiles_workspace_floats(rows, r);
   return gram_slices(rows) * (int64_t)gram_pairs(r) * 1024;
 }
 
@@ -359,6 +362,8 @@ __global__ void __launch_bounds__(256)
 
 int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace) {
   DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
+  if (gram_uses_tiles(rows, r) && ((uintptr_t)X % 16) == 0)
+    return launch_gram_tiles(rows, r, X, G, workspace);
   const int n_pairs = gram_pairs(r);
   const int n_tiles = (r + 127) / 128;
   int64_t slices = gram_slices(rows);

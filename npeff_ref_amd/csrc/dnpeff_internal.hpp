@@ -86,6 +86,9 @@ int launch_mu(int64_t count, float* F, const float* num, const float* den, float
 // Needs a workspace of gram_workspace_floats(rows, r) floats.
 int64_t gram_workspace_floats(int64_t rows, int r);
 int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace);
+// ranks 256, 384, ..., 1024 (head.hip)
+int64_t gram_tiles_workspace_floats(int64_t rows, int r);
+int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace);
 int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const float* num, float eps,
                  float* out, float* D_out);
 // dot with fp64 accumulation; result lands in *out_dev (one double, device).

@@ -38,8 +38,10 @@ struct PtqStage {
 
 __global__ void __launch_bounds__(256)
     k_ptq(const float* __restrict__ P, int64_t ldp, int64_t K, const float* __restrict__ Q, int r,
-          int64_t M, int64_t M_pad, int64_t tiles_per_slice, float* __restrict__ out) {
+          int64_t M, int64_t M_pad, int64_t tiles_per_slice, int upper_only,
+          float* __restrict__ out) {
   extern __shared__ __align__(16) float lds[];  // 2 * PTQ_SLOT floats
+  if (upper_only && blockIdx.x > blockIdx.y) return;  // symmetric product: tiles (i <= j) only
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
@@ -158,7 +160,7 @@ static int64_t ptq_slices(int64_t tiles_mn, int64_t k_tiles) {
 }
 
 static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, int r, int64_t M,
-                      int64_t M_pad, int64_t slices, float* out) {
+                      int64_t M_pad, int64_t slices, float* out, int upper_only = 0) {
   static bool attr_set = false;
   const size_t lds = sizeof(float) * 2 * PTQ_SLOT;
   if (!attr_set) {
@@ -171,7 +173,47 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
   DN_CHECK(M_pad % 128 == 0 && ldp % 4 == 0 && r % 4 == 0, "dense product: misaligned operands");
   DN_CHECK(M_pad / 128 < ((int64_t)1 << 22), "dense product: too many row tiles");
   dim3 grid((unsigned)(M_pad / 128), (unsigned)ceil_div(r, 128), (unsigned)slices);
-  hipLaunchKernelGGL(k_ptq, grid, dim3(256), lds, stream(), P, ldp, K, Q, r, M, M_pad, per, out);
+  hipLaunchKernelGGL(k_ptq, grid, dim3(256), lds, stream(), P, ldp, K, Q, r, M, M_pad, per,
+                     upper_only, out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Gram X^T X for ranks that are multiples of 128 above 128: the same tiles with P = Q = X, only
+// the tile pairs (i <= j), K split into slices; the reduction sums the slices in fp64 and writes
+// every element and its mirror image.
+// ---------------------------------------------------------------------------
+static int64_t gram_tiles_slices(int64_t rows, int r) {
+  const int64_t t = r / 128, pairs = t * (t + 1) / 2;
+  int64_t s = ceil_div(1024, pairs);
+  const int64_t k_tiles = ceil_div(rows, PTQ_KB);
+  if (s > k_tiles) s = k_tiles;
+  return s < 1 ? 1 : s;
+}
+
+int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
+  return gram_tiles_slices(rows, r) * (int64_t)r * r;
+}
+
+__global__ void __launch_bounds__(256)
+    k_gram_tiles_reduce(const float* __restrict__ ws, int64_t slices, int r, float* __restrict__ G) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= r * r) return;
+  const int a = e / r, b = e % r;
+  if ((a >> 7) > (b >> 7) || ((a >> 7) == (b >> 7) && a > b)) return;  // upper triangle only
+  double s = 0.0;
+  const int64_t stride = (int64_t)r * r;
+  for (int64_t sl = 0; sl < slices; sl++) s += (double)ws[sl * stride + e];
+  G[(int64_t)a * r + b] = (float)s;
+  G[(int64_t)b * r + a] = (float)s;
+}
+
+int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace) {
+  const int64_t slices = gram_tiles_slices(rows, r);
+  DN_TRY(launch_ptq(X, r, rows, X, r, r, r, slices, workspace, 1));
+  hipLaunchKernelGGL(k_gram_tiles_reduce, dim3((unsigned)ceil_div((int64_t)r * r, 256)), dim3(256), 0,
+                     stream(), workspace, slices, r, G);
   DN_LAUNCH_CHECK();
   return 0;
 }
