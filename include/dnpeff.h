@@ -302,6 +302,14 @@ int dnpeff_op_spmm_n(dnpeff_csr* A, int r, const float* H_mr, float* N_nr);
  * cusparseSpMM(T, T) at device_contexts1.h:260-265,301. */
 int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 
+/* Keeps the elements with x[i] / divisor >= threshold (fp32 division, then the comparison):
+ * idx_out receives their positions in ascending order, val_out the divided values, *n_kept
+ * (host) their number; idx_out and val_out are device buffers of `count` elements.  One row of
+ * the dense-to-sparse conversion of H, to_csr in scripts/sparsify_d_npeff.py:27-49, after the
+ * row has been scaled to unit norm (:56). */
+int dnpeff_op_threshold_compact(int64_t count, const float* x, float divisor, float threshold,
+                                int32_t* idx_out, float* val_out, int64_t* n_kept);
+
 /* G[r, r] = X^T X for X [rows, r].  cublasSgemm at device_contexts1.h:303,322. */
 int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr);
 

@@ -29,6 +29,7 @@ from .binding import (  # noqa: F401
     device_info,
     op_mu,
     op_spmm_n,
+    op_threshold_compact,
     op_spmm_t,
     op_gram,
     op_xg_mu,

@@ -60,6 +60,7 @@ SIGNATURES = {
     "dnpeff_csr_kept_indices": (C.c_int, [_p, _p]),
     "dnpeff_csr_sq_norm": (C.c_int, [_p, C.POINTER(_f64)]),
     "dnpeff_csr_build_transpose": (C.c_int, [_p]),
+    "dnpeff_op_threshold_compact": (C.c_int, [C.c_int64, _p, C.c_float, C.c_float, _p, _p, C.POINTER(C.c_int64)]),
     "dnpeff_csr_split_dense_head": (C.c_int, [_p, C.c_double, C.POINTER(C.c_int64)]),
     "dnpeff_csr_head_info": (C.c_int, [_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "dnpeff_csr_download_transpose": (C.c_int, [_p, _p, _p, _p]),
@@ -239,6 +240,17 @@ def op_spsp_dense(A: "Csr", B: "Csr", out: DeviceArray):
 
 def op_init_uniform(matrix_id: int, logical_rows: int, logical_cols: int, seed: int, x: DeviceArray):
     _check(lib.dnpeff_op_init_uniform(matrix_id, logical_rows, logical_cols, seed & 0xFFFFFFFFFFFFFFFF, x.ptr))
+
+
+def op_threshold_compact(x: "DeviceArray", divisor: float, threshold: float):
+    """(positions, values) of the elements with x / divisor >= threshold, as numpy arrays."""
+    n = int(np.prod(x.shape))
+    idx = DeviceArray((max(n, 1),), dtype=np.int32)
+    val = DeviceArray((max(n, 1),), dtype=np.float32)
+    kept = _i64(0)
+    _check(lib.dnpeff_op_threshold_compact(n, x.ptr, float(divisor), float(threshold), idx.ptr, val.ptr,
+                                           C.byref(kept)))
+    return idx.numpy()[:kept.value].copy(), val.numpy()[:kept.value].copy()
 
 
 class Csr:

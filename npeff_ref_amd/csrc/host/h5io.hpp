@@ -258,6 +258,19 @@ inline DenseDecomposition read_dense_decomposition(const std::string& path) {
   return d;
 }
 
+// Rows [row0, row0 + n_rows) of a 2-D float dataset.
+inline void read_rows_2d(hid_t file, const char* name, long row0, long n_rows, long n_cols, float* out) {
+  hid_t ds = check(H5Dopen(file, name, H5P_DEFAULT), std::string("open ") + name);
+  hid_t sp = H5Dget_space(ds);
+  hsize_t start[2] = {(hsize_t)row0, 0}, count[2] = {(hsize_t)n_rows, (hsize_t)n_cols};
+  hid_t mem = H5Screate_simple(2, count, count);
+  check_status(H5Sselect_hyperslab(sp, H5S_SELECT_SET, start, nullptr, count, nullptr), "hyperslab");
+  check_status(H5Dread(ds, H5T_NATIVE_FLOAT, mem, sp, H5P_DEFAULT, out), std::string("read ") + name);
+  H5Sclose(mem);
+  H5Sclose(sp);
+  H5Dclose(ds);
+}
+
 struct SparseDecomposition {
   long n = 0, r = 0, m = 0;            // W [n, r]; H [r, m] CSR
   std::vector<float> W;

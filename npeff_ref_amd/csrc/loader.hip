@@ -171,6 +171,12 @@ struct LongColF {
   }
 };
 
+struct GeThresholdF {
+  const float* x;
+  float divisor, threshold;
+  __device__ int64_t operator()(int64_t i) const { return x[i] / divisor >= threshold ? 1 : 0; }
+};
+
 int scan_keep_mask(const int* count, int min_count, int64_t n, int32_t* out) {
   return exclusive_scan(KeepMaskF{count, min_count}, n, out);
 }
@@ -356,6 +362,21 @@ __global__ void __launch_bounds__(256)
         }
       }
       __syncthreads();
+    }
+  }
+}
+
+// idx_out / val_out [pos[i]] = (i, x[i] / divisor) for the elements that pass the threshold
+__global__ void __launch_bounds__(256)
+    k_threshold_write(const float* __restrict__ x, float divisor, float threshold, int64_t n,
+                      const int64_t* __restrict__ pos, int32_t* __restrict__ idx_out,
+                      float* __restrict__ val_out) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const float v = x[i] / divisor;
+    if (v >= threshold) {
+      idx_out[pos[i]] = (int32_t)i;
+      val_out[pos[i]] = v;
     }
   }
 }
@@ -992,6 +1013,32 @@ DN_API int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* 
   A->tail = T;
   if (n_dense) *n_dense = n_d;
   return 0;
+}
+
+DN_API int dnpeff_op_threshold_compact(int64_t count, const float* x, float divisor, float threshold,
+                                       int32_t* idx_out, float* val_out, int64_t* n_kept) {
+  clear_error();
+  DN_CHECK(count >= 0 && count <= (int64_t)INT32_MAX, "count %lld outside [0, 2^31)", (long long)count);
+  DN_CHECK((x && idx_out && val_out) || count == 0, "NULL argument");
+  DN_CHECK(n_kept != nullptr, "n_kept is NULL");
+  DN_CHECK(divisor != 0.0f, "divisor is zero");
+  *n_kept = 0;
+  if (count == 0) return 0;
+  int64_t* pos = nullptr;
+  DN_TRY(dmalloc(&pos, count + 1));
+  int s = exclusive_scan(GeThresholdF{x, divisor, threshold}, count, pos);
+  if (!s) {
+    hipLaunchKernelGGL(k_threshold_write, dim3(grid_for(count)), dim3(256), 0, stream(), x, divisor,
+                       threshold, count, pos, idx_out, val_out);
+    if (hipGetLastError() != hipSuccess ||
+        hipMemcpy(n_kept, pos + count, sizeof(int64_t), hipMemcpyDeviceToHost) != hipSuccess) {
+      set_error("threshold compaction failed");
+      s = 1;
+    }
+  }
+  (void)hipStreamSynchronize(stream());
+  dfree(pos);
+  return s;
 }
 
 DN_API int dnpeff_csr_head_info(const dnpeff_csr* A, int64_t* n_dense, int64_t* nnz_sparse) {

@@ -262,6 +262,28 @@ class F32Baseline:
 
 
 # ---- compiled reference routines (oracle/_ref) ----------------------------------------------
+def sparsify_H(W, H_rm, threshold):
+    """Dense decomposition -> (W', values, row_offsets, column_indices): every row of H scaled to
+    unit L2 norm (sum of squares in fp64, norm and division in fp32), the matching column of W
+    multiplied by the norm, then per row the entries >= threshold in ascending column order.
+    scripts/sparsify_d_npeff.py:27-49 (to_csr) and :56 (the normalisation it intends)."""
+    H = np.asarray(H_rm, dtype=np.float32)
+    W2 = np.array(W, dtype=np.float32, copy=True)
+    thr = np.float32(threshold)
+    vals, cols, offs = [], [], [0]
+    for k in range(H.shape[0]):
+        norm = np.float32(np.sqrt(np.sum(H[k].astype(np.float64) ** 2)))
+        div = norm if norm > 0 else np.float32(1.0)
+        row = (H[k] / div).astype(np.float32)
+        mask = row >= thr
+        vals.append(row[mask])
+        cols.append(np.nonzero(mask)[0].astype(np.int32))
+        offs.append(offs[-1] + int(mask.sum()))
+        W2[:, k] *= div
+    return (W2, np.concatenate(vals).astype(np.float32), np.array(offs, dtype=np.int64),
+            np.concatenate(cols).astype(np.int32))
+
+
 def have_ref():
     return _ref is not None
 

@@ -292,3 +292,14 @@ def test_column_panels_with_dense_head(monkeypatch):
     N64 = orc.spmm_n_f64(rp, ci, va, H)
     assert (np.abs(dN.numpy() - N64).max(axis=1) / np.abs(N64).max(axis=1)).max() < TOL
     A.close()
+
+
+@pytest.mark.parametrize("n,div,thr", [(100003, 3.7, 0.1), (5, 1.0, 0.0), (4096, 0.5, 5.0), (70000, 2.0, -1.0)])
+def test_threshold_compact_bit_exact(n, div, thr):
+    rng = np.random.default_rng(n)
+    x = rng.random(n).astype(np.float32)
+    idx, val = d.op_threshold_compact(d.DeviceArray.from_numpy(x), div, thr)
+    q = (x / np.float32(div)).astype(np.float32)
+    keep = q >= np.float32(thr)
+    assert np.array_equal(idx, np.nonzero(keep)[0].astype(np.int32))
+    assert np.array_equal(val, q[keep])

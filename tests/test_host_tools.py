@@ -166,3 +166,38 @@ def test_fit_row_split_check_is_kept(tmp_path):
     assert "NOTE: Using flag intended only for development purposes." in p.stdout
     shape_attr, _ = h5lite.attr(f"{tmp_path}/o.h5", "data/H", "shape")
     assert shape_attr.tolist() == [4, 1000]
+
+
+@pytest.mark.gpu
+def test_sparsify_d_npeff_feeds_the_fit(tmp_path):
+    """run_nmf_on_pefs -> sparsify_d_npeff -> fit_coeffs_to_sparse_H: the sparsifier's file has the
+    sparse schema with unit-norm thresholded rows of H and rescaled W, and the fit accepts it."""
+    n, m_full, k, r = 40, 30000, 500, 8
+    pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=5)
+    dense, sparse, fit = (str(tmp_path / f) for f in ("decomp.h5", "sparse.h5", "fit.h5"))
+    run("run_nmf_on_pefs", f"--output_path={dense}", f"--per_example_fishers={pef}", f"--nmf_n_components={r}",
+        "--nmf_max_iter=30", check=True)
+    thr = 0.004
+    p = run("sparsify_d_npeff", f"--decomposition_filepath={dense}", f"--output_filepath={sparse}",
+            f"--H_threshold={thr}", check=True)
+    W, H = h5lite.read(dense, "data/W"), h5lite.read(dense, "data/H")
+    W2, vals, offs, cols = orc.sparsify_H(W, H, thr)
+    assert f"Dense size: {H.size}" in p.stdout and f"Sparse NNZ: {len(vals)}" in p.stdout
+    assert 0 < len(vals) < H.size
+    assert np.array_equal(h5lite.read(sparse, "data/H/values"), vals)
+    assert np.array_equal(h5lite.read(sparse, "data/H/column_indices"), cols)
+    got_offs = h5lite.read(sparse, "data/H/row_indices")
+    assert got_offs.dtype == np.int64 and np.array_equal(got_offs, offs)
+    assert np.array_equal(h5lite.read(sparse, "data/W"), W2)
+    assert np.array_equal(h5lite.read(sparse, "data/reduce_kept_indices"), h5lite.read(dense, "data/reduce_kept_indices"))
+    shape_attr, _ = h5lite.attr(sparse, "data/H", "shape")
+    assert shape_attr.tolist() == list(H.shape)
+    fds, _ = h5lite.attr(sparse, "data/reduce_kept_indices", "full_dense_size")
+    assert int(fds[0]) == m_full
+    # missing threshold is fatal, as the script's assert
+    q = run("sparsify_d_npeff", f"--decomposition_filepath={dense}", f"--output_filepath={sparse}.x")
+    assert q.returncode != 0 and "Missing flag: H_threshold" in q.stdout
+    # the other executable takes the file
+    run("fit_coeffs_to_sparse_H", f"--output_path={fit}", f"--pef_path={pef}", f"--H_path={sparse}",
+        "--n_splits_sparse_matmul=1", "--n_row_splits_pefs=1", "--nmf_max_iter=25", check=True)
+    assert h5lite.read(fit, "data/W").shape == (n, r)

@@ -137,3 +137,29 @@ def test_f32_baseline_tracks_f64_oracle():
     b.close()
     assert np.linalg.norm(W32 - W64) / np.linalg.norm(W64) < 1e-5
     assert np.linalg.norm(H32 - H64) / np.linalg.norm(H64) < 1e-5
+
+
+def test_sparsify_H_keeps_the_product_and_thresholds_unit_norm_rows():
+    """The product W H is unchanged by the normalisation, kept rows have unit norm, threshold 0
+    on non-negative H keeps every entry, and a dense rebuild of the CSR equals the thresholded
+    unit-norm H (to_csr of scripts/sparsify_d_npeff.py:27-49 written out densely)."""
+    rng = np.random.default_rng(9)
+    r, m, n = 5, 300, 7
+    H = (rng.random((r, m)) * (rng.random((r, m)) < 0.3)).astype(np.float32)
+    H[3] = 0.0  # a dead component stays as it is
+    W = rng.random((n, r)).astype(np.float32)
+    W2, vals, offs, cols = orc.sparsify_H(W, H, 0.0)
+    assert offs[-1] == r * m and np.array_equal(cols[:m], np.arange(m))
+    Hn = vals.reshape(r, m)
+    assert np.allclose(W2.astype(np.float64) @ Hn, W.astype(np.float64) @ H, rtol=1e-5, atol=1e-7)
+    norms = np.linalg.norm(Hn.astype(np.float64), axis=1)
+    assert np.allclose(norms[[0, 1, 2, 4]], 1.0, atol=1e-6) and norms[3] == 0
+    thr = 0.08
+    W3, vals, offs, cols = orc.sparsify_H(W, H, thr)
+    dense = np.zeros((r, m), np.float32)
+    for k in range(r):
+        c = cols[offs[k]:offs[k + 1]]
+        assert np.all(np.diff(c) > 0)
+        dense[k, c] = vals[offs[k]:offs[k + 1]]
+    assert np.array_equal(dense, np.where(Hn >= np.float32(thr), Hn, 0).astype(np.float32))
+    assert np.array_equal(W3, W2)
