@@ -29,7 +29,9 @@ typedef float acc16 __attribute__((ext_vector_type(16)));
 // free.  Wave (wm, wn) owns blocks {2 wm, 2 wm + 1} x {2 wn, 2 wn + 1}.
 // ---------------------------------------------------------------------------
 constexpr int PTQ_KB = 32;
-constexpr int PTQ_HALF = PTQ_KB * 128;   // floats of one operand tile
+constexpr int PTQ_LD = 160;              // LDS row: 128 floats + 32, so that the two half-waves
+                                         // (rows k and k + 1) fall on different banks
+constexpr int PTQ_HALF = PTQ_KB * PTQ_LD;  // floats of one operand tile
 constexpr int PTQ_SLOT = 2 * PTQ_HALF;   // floats of one slot
 
 struct PtqStage {
@@ -38,7 +40,7 @@ struct PtqStage {
 
 __global__ void __launch_bounds__(256)
     k_ptq(const float* __restrict__ P, int64_t ldp, int64_t K, const float* __restrict__ Q, int r,
-          int64_t M, int64_t M_pad, int64_t tiles_per_slice, int upper_only,
+          int64_t M, int64_t M_pad, int upper_only,
           float* __restrict__ out) {
   extern __shared__ __align__(16) float lds[];  // 2 * PTQ_SLOT floats
   if (upper_only && blockIdx.x > blockIdx.y) return;  // symmetric product: tiles (i <= j) only
@@ -47,11 +49,11 @@ __global__ void __launch_bounds__(256)
   const int wm = wave >> 1, wn = wave & 1;
   const int64_t m0 = (int64_t)blockIdx.x * 128;
   const int n0 = blockIdx.y * 128;
+  // the K tiles are dealt to the slices round-robin (slice z owns tiles z, z + S, ...), so that
+  // at any moment the workgroups read one contiguous window of P and Q
   const int64_t all_tiles = (K + PTQ_KB - 1) / PTQ_KB;
-  const int64_t t0 = (int64_t)blockIdx.z * tiles_per_slice;
-  int64_t n_tiles = all_tiles - t0;
-  if (n_tiles > tiles_per_slice) n_tiles = tiles_per_slice;
-  if (n_tiles < 0) n_tiles = 0;
+  const int64_t S = gridDim.z, z = blockIdx.z;
+  const int64_t n_tiles = all_tiles > z ? (all_tiles - z + S - 1) / S : 0;
 
   // loader role of a thread: 16-byte column li of rows lr + 8 q of a tile
   const int li = threadIdx.x & 31, lr = threadIdx.x >> 5;
@@ -60,7 +62,7 @@ __global__ void __launch_bounds__(256)
   const float* pQ = Q + n0 + 4 * li;
 
   auto fetch = [&](PtqStage& s, int64_t tile) {
-    const int64_t kbase = (t0 + tile) * PTQ_KB + lr;
+    const int64_t kbase = (z + tile * S) * PTQ_KB + lr;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       const int64_t k = kbase + 8 * q;
@@ -74,7 +76,7 @@ __global__ void __launch_bounds__(256)
   auto commit = [&](const PtqStage& s, float* slot) {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-      float* a = slot + (lr + 8 * q) * 128 + li;
+      float* a = slot + (lr + 8 * q) * PTQ_LD + li;
       a[0] = s.p[q].x; a[32] = s.p[q].y; a[64] = s.p[q].z; a[96] = s.p[q].w;
       float* b = a + PTQ_HALF;
       b[0] = s.q[q].x; b[32] = s.q[q].y; b[64] = s.q[q].z; b[96] = s.q[q].w;
@@ -90,18 +92,18 @@ __global__ void __launch_bounds__(256)
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
   auto mfma_slot = [&](const float* slot) {
-    const float* pa = slot + half * 128 + 64 * wm + l32;
-    const float* pb = slot + PTQ_HALF + half * 128 + 64 * wn + l32;
+    const float* pa = slot + half * PTQ_LD + 64 * wm + l32;
+    const float* pb = slot + PTQ_HALF + half * PTQ_LD + 64 * wn + l32;
     constexpr int GRP = 4;
 #pragma unroll
     for (int g = 0; g < PTQ_KB / 2; g += GRP) {
       float xa[GRP][2], xb[GRP][2];
 #pragma unroll
       for (int u = 0; u < GRP; u++) {
-        xa[u][0] = pa[2 * (g + u) * 128];
-        xa[u][1] = pa[2 * (g + u) * 128 + 32];
-        xb[u][0] = pb[2 * (g + u) * 128];
-        xb[u][1] = pb[2 * (g + u) * 128 + 32];
+        xa[u][0] = pa[2 * (g + u) * PTQ_LD];
+        xa[u][1] = pa[2 * (g + u) * PTQ_LD + 32];
+        xb[u][0] = pb[2 * (g + u) * PTQ_LD];
+        xb[u][1] = pb[2 * (g + u) * PTQ_LD + 32];
       }
 #pragma unroll
       for (int u = 0; u < GRP; u++)
@@ -153,7 +155,7 @@ __global__ void __launch_bounds__(256)
 
 // slices of K so that the launch holds about a thousand workgroups
 static int64_t ptq_slices(int64_t tiles_mn, int64_t k_tiles) {
-  int64_t s = 1024 / (tiles_mn > 0 ? tiles_mn : 1);
+  int64_t s = (4 * (int64_t)n_cus()) / (tiles_mn > 0 ? tiles_mn : 1);
   if (s > 64) s = 64;
   if (s > k_tiles) s = k_tiles;
   return s < 1 ? 1 : s;
@@ -168,12 +170,10 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
-  const int64_t k_tiles = ceil_div(K, PTQ_KB);
-  const int64_t per = ceil_div(k_tiles, slices);
   DN_CHECK(M_pad % 128 == 0 && ldp % 4 == 0 && r % 4 == 0, "dense product: misaligned operands");
   DN_CHECK(M_pad / 128 < ((int64_t)1 << 22), "dense product: too many row tiles");
   dim3 grid((unsigned)(M_pad / 128), (unsigned)ceil_div(r, 128), (unsigned)slices);
-  hipLaunchKernelGGL(k_ptq, grid, dim3(256), lds, stream(), P, ldp, K, Q, r, M, M_pad, per,
+  hipLaunchKernelGGL(k_ptq, grid, dim3(256), lds, stream(), P, ldp, K, Q, r, M, M_pad,
                      upper_only, out);
   DN_LAUNCH_CHECK();
   return 0;
@@ -186,7 +186,8 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
 // ---------------------------------------------------------------------------
 static int64_t gram_tiles_slices(int64_t rows, int r) {
   const int64_t t = r / 128, pairs = t * (t + 1) / 2;
-  int64_t s = ceil_div(1024, pairs);
+  // two workgroups fit a CU: at most 2 rounds of 2 x 256 workgroups, never a few stragglers
+  int64_t s = (4 * (int64_t)n_cus()) / pairs;
   const int64_t k_tiles = ceil_div(rows, PTQ_KB);
   if (s > k_tiles) s = k_tiles;
   return s < 1 ? 1 : s;

@@ -180,3 +180,40 @@ def test_column_panel_run_matches_oracle(monkeypatch):
     assert np.all(np.abs(got - losses64) / losses64 < REL)
     nmf.close()
     A.close()
+
+
+def test_ragged_rows_rank_512(monkeypatch):
+    """Row lengths drawn log-uniformly over two decades (the ragged-row case), r = 512: the tiled
+    X G kernel, the tile-pair Gram and the grouped A^T W at their widest, with column panels
+    forced on so that short rows leave empty segments."""
+    monkeypatch.setenv("DNPEFF_PANELS", "24")
+    n, m_full, r, eps, iters, seed = 260, 60000, 512, 1e-8, 50, 31
+    A, norms = d.Csr.synth(n, m_full, k_fixed=0, k_min=16, k_max=4096, zipf_s=1.1, seed=seed)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    rp, ci, va = A.download()
+    lens = np.diff(rp)
+    assert lens.min() < 64 and lens.max() > 2000
+    m = A.n_cols
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=iters, eps=eps, seed=seed, log_every=10))
+    nmf.initialize()
+    W0, H0 = nmf.loadWToHostSync(), nmf.loadHToHostSync()
+    hist = nmf.run(log=lambda s: None)
+    W64, H64, losses64 = orc.nmf_f64(rp, ci, va, m, W0, H0, np.float32(eps), iters, 10)
+    assert _nrm(nmf.loadWToHostSync(), W64) < REL and _nrm(nmf.loadHToHostSync(), H64) < REL
+    got = np.array([h[1] for h in hist])
+    assert np.all(np.abs(got - losses64) / losses64 < REL)
+    nmf.close()
+    A.close()
+
+
+def test_heavier_skew_rank_256_with_dense_head():
+    """Zipf 1.3 columns, r = 256, enough rows for the dense head: every r > 128 kernel plus the
+    head products in one run."""
+    nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(1030, 200000, 1500, 256, 1e-8, 50, seed=13, zipf_s=1.3)
+    assert A.head_info()[0] > 50
+    assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
+    got = np.array([h[1] for h in hist])
+    assert np.all(np.abs(got - losses64) / losses64 < REL)
+    nmf.close()
+    A.close()
