@@ -22,11 +22,11 @@ typedef float acc16 __attribute__((ext_vector_type(16)));
 //
 // A workgroup of 4 waves owns a 128 x 128 tile of C and a contiguous range of K, streamed in
 // tiles of 32 contraction rows through two LDS slots (P tile then Q tile, 16 KB each), fetched
-// with 16-byte loads two tiles ahead into registers.  v_mfma_f32_32x32x2f32 takes from lane l
-// A[i = l%32][k = l/32] and B[k = l/32][j = l%32]; the 32 rows (columns) of an operand block are
-// every fourth element of the 128-wide tile (block a holds 4 i + a), stored in LDS as four runs
-// of 32 floats, so one 16-byte global load feeds four blocks and every LDS read is conflict
-// free.  Wave (wm, wn) owns blocks {2 wm, 2 wm + 1} x {2 wn, 2 wn + 1}.
+// with 16-byte loads two tiles ahead into registers and written to LDS as they are (16-byte
+// stores).  v_mfma_f32_32x32x2f32 takes from lane l A[i = l%32][k = l/32] and
+// B[k = l/32][j = l%32]: a lane reads P[k][32 a + i] and Q[k][32 b + j] of its blocks with 4-byte
+// LDS reads, the two half-waves on rows k and k + 1.  Wave (wm, wn) owns the 32-wide blocks
+// {2 wm, 2 wm + 1} x {2 wn, 2 wn + 1} of the tile.
 // ---------------------------------------------------------------------------
 constexpr int PTQ_KB = 32;
 constexpr int PTQ_LD = 160;              // LDS row: 128 floats + 32, so that the two half-waves
@@ -76,10 +76,9 @@ __global__ void __launch_bounds__(256)
   auto commit = [&](const PtqStage& s, float* slot) {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-      float* a = slot + (lr + 8 * q) * PTQ_LD + li;
-      a[0] = s.p[q].x; a[32] = s.p[q].y; a[64] = s.p[q].z; a[96] = s.p[q].w;
-      float* b = a + PTQ_HALF;
-      b[0] = s.q[q].x; b[32] = s.q[q].y; b[64] = s.q[q].z; b[96] = s.q[q].w;
+      float* a = slot + (lr + 8 * q) * PTQ_LD + 4 * li;
+      *reinterpret_cast<float4*>(a) = s.p[q];
+      *reinterpret_cast<float4*>(a + PTQ_HALF) = s.q[q];
     }
   };
 
@@ -91,27 +90,37 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+  // Operands of 4 row pairs are read one group ahead of the MFMAs that use them; the scheduling
+  // fences keep the compiler from sinking the LDS reads back to their first use, which would
+  // expose the LDS latency once per 4 MFMAs.
   auto mfma_slot = [&](const float* slot) {
     const float* pa = slot + half * PTQ_LD + 64 * wm + l32;
     const float* pb = slot + PTQ_HALF + half * PTQ_LD + 64 * wn + l32;
-    constexpr int GRP = 4;
-#pragma unroll
-    for (int g = 0; g < PTQ_KB / 2; g += GRP) {
-      float xa[GRP][2], xb[GRP][2];
+    constexpr int GRP = 4, NG = PTQ_KB / 2 / GRP;
+    float xa[2][GRP][2], xb[2][GRP][2];
+    auto read_group = [&](int g, float (&ya)[GRP][2], float (&yb)[GRP][2]) {
 #pragma unroll
       for (int u = 0; u < GRP; u++) {
-        xa[u][0] = pa[2 * (g + u) * PTQ_LD];
-        xa[u][1] = pa[2 * (g + u) * PTQ_LD + 32];
-        xb[u][0] = pb[2 * (g + u) * PTQ_LD];
-        xb[u][1] = pb[2 * (g + u) * PTQ_LD + 32];
+        ya[u][0] = pa[2 * (g * GRP + u) * PTQ_LD];
+        ya[u][1] = pa[2 * (g * GRP + u) * PTQ_LD + 32];
+        yb[u][0] = pb[2 * (g * GRP + u) * PTQ_LD];
+        yb[u][1] = pb[2 * (g * GRP + u) * PTQ_LD + 32];
       }
+    };
+    read_group(0, xa[0], xb[0]);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+      if (g + 1 < NG) read_group(g + 1, xa[(g + 1) & 1], xb[(g + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int u = 0; u < GRP; u++)
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
           for (int j = 0; j < 2; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u][i], xb[u][j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[g & 1][u][i], xb[g & 1][u][j],
+                                                             acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
@@ -136,19 +145,17 @@ __global__ void __launch_bounds__(256)
   if (t < n_tiles) mfma_slot(lds);
 
   // D layout of a 32x32 block: reg v of lane l holds row 8 (v/4) + 4 (l/32) + v%4, column l%32;
-  // block (a, b) row ib is C row 4 ib + a, column jb is C column 4 jb + b.  The wave's two
-  // column blocks are adjacent columns: one 8-byte store.
-  const int n = 4 * l32 + 2 * wn;
-  if (n0 + n < r) {
-    float* base = out + ((int64_t)blockIdx.z * M_pad + m0) * r + n0 + n;
+  // block (i, j) of the wave covers rows 64 wm + 32 i.., columns 64 wn + 32 j.. of the tile.
+  float* base = out + ((int64_t)blockIdx.z * M_pad + m0 + 64 * wm + 4 * half) * r + n0 + 64 * wn + l32;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    if (n0 + 64 * wn + 32 * j + l32 >= r) continue;
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const int ib = 8 * (v >> 2) + 4 * half + (v & 3);
-        const int m = 4 * ib + 2 * wm + i;
-        if (m0 + m < M)
-          *reinterpret_cast<float2*>(base + (int64_t)m * r) = make_float2(acc[i][0][v], acc[i][1][v]);
+        const int below = 32 * i + 8 * (v >> 2) + (v & 3);
+        if (m0 + 64 * wm + 4 * half + below < M) base[(int64_t)below * r + 32 * j] = acc[i][j][v];
       }
   }
 }

@@ -718,10 +718,12 @@ DN_API int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr
 DN_API int dnpeff_op_spsp_dense(dnpeff_csr* A, dnpeff_csr* B, float* out_nr) {
   clear_error();
   DN_CHECK(A && B && out_nr, "NULL argument");
+  // this product walks the plain CSR structures: a split left by an earlier NMF is undone
+  if (A->tail) DN_TRY(dnpeff_csr_split_dense_head(A, 0.0, nullptr));
+  if (B->tail) DN_TRY(dnpeff_csr_split_dense_head(B, 0.0, nullptr));
   DN_TRY(dnpeff_csr_build_transpose(B));
   const int r = (int)B->n_rows;
   DN_TRY(csr_ensure_partials(A, r));
-  DN_CHECK(!A->tail && !B->tail, "sparse-sparse product of matrices with a dense head");
   DN_TRY(launch_spsp(A, B, A->partials));
   return launch_chunk_reduce(A, r, A->partials, out_nr);
 }

@@ -217,3 +217,30 @@ def test_heavier_skew_rank_256_with_dense_head():
     assert np.all(np.abs(got - losses64) / losses64 < REL)
     nmf.close()
     A.close()
+
+
+def test_fit_after_nmf_on_the_same_matrix():
+    """A matrix that an NMF has split (dense head, tail) is handed to the fit path afterwards:
+    the sparse-sparse product undoes the split and gives the same A H^T as on a fresh matrix."""
+    n, m_full, k, r = 1100, 60000, 3000, 64
+    A, norms = d.Csr.synth(n, m_full, k_fixed=k, zipf_s=1.1, seed=77)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    rp, ci, va = A.download()
+    m = A.n_cols
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=2, eps=1e-8, seed=1))
+    nmf.initialize()
+    nmf.run(log=lambda s: None)
+    assert A.head_info()[0] > 0
+    nmf.close()
+    rng = np.random.default_rng(0)
+    hr, hc, hv = random_csr(rng, 8, m, 300, sort_cols=True)
+    B = d.Csr.from_host(hr, hc, hv, m)
+    out = d.DeviceArray((n, 8))
+    d.op_spsp_dense(A, B, out)
+    assert A.head_info()[0] == 0
+    want = orc.spsp_dense_f64((rp, ci, va), m, (hr, hc, hv), 8)
+    got = out.numpy()
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+    A.close()
+    B.close()
