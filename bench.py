@@ -51,8 +51,9 @@ def log(msg):
     print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
 
 
-def algorithmic(cls, n, m, z, r):
-    """Compulsory traffic / flops of one launch: every operand touched once."""
+def algorithmic(cls, n, m, z, r, fused_gram=False):
+    """Compulsory traffic / flops of one launch: every operand touched once.  With fused_gram the
+    H update also produces H^T H (no separate gram_H launch): its class carries both products."""
     P = 4 if z < 2**31 else 8
     if cls == "spmm_n":
         return "hbm", 8 * z + P * (n + 1) + 4 * r * m + 4 * n * r
@@ -65,6 +66,8 @@ def algorithmic(cls, n, m, z, r):
     if cls == "gram_W":
         return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 4 * n * r + 4 * r * r)
     if cls == "xg_mu_H":
+        if fused_gram:
+            return "mfma", 4 * m * r * r
         return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 12 * m * r + 4 * r * r)
     if cls == "xg_mu_W":
         return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 12 * n * r + 4 * r * r)
@@ -170,10 +173,11 @@ def main():
     log(f"{args.steps} steps in {elapsed:.3f} s -> {ms_per_step:.2f} ms/step, loss {loss:.10g}")
 
     kernels = {}
+    fused_gram = tim.get("gram_H", (0.0, 0))[1] == 0
     for cls, (ms_sum, cnt) in tim.items():
         if cnt == 0:
             continue
-        bound, work = algorithmic(cls, n, m, z, r)
+        bound, work = algorithmic(cls, n, m, z, r, fused_gram)
         avg_s = ms_sum / cnt * 1e-3
         peak = HBM_PEAK if bound == "hbm" else MFMA_FP32_PEAK
         kernels[cls] = dict(
@@ -213,6 +217,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "kernels": kernels,
+        "fused_gram_in_H_update": fused_gram,
         "spmm_hbm_frac": {k: kernels[k]["frac"] for k in ("spmm_n", "spmm_t") if k in kernels},
         "loss_after": loss,
     }

@@ -87,6 +87,9 @@ struct dnpeff_nmf {
   float* G2 = nullptr;       // [r, r]
   float* gram_ws = nullptr;  // slice partials of the Gram kernel
   double* dot_ws = nullptr;  // DOT_BLOCKS partials + 2 results
+  float* GH = nullptr;       // [r, r] H^T H from the fused H update (valid while gh_valid)
+  float* gpart = nullptr;    // its partial sums
+  bool gh_valid = false;
   double sq_norm_A = 0.0;
   Profiler prof;
 };
@@ -96,6 +99,7 @@ DN_API int dnpeff_nmf_destroy(dnpeff_nmf* nmf) {
   (void)hipStreamSynchronize(stream());
   dfree(nmf->W); dfree(nmf->W2); dfree(nmf->Nw); dfree(nmf->H); dfree(nmf->S);
   dfree(nmf->G); dfree(nmf->G2); dfree(nmf->gram_ws); dfree(nmf->dot_ws);
+  dfree(nmf->GH); dfree(nmf->gpart);
   delete nmf;
   return 0;
 }
@@ -116,6 +120,14 @@ static int default_head_split(dnpeff_csr* A, int rank) {
     return 0;
   }
   return dnpeff_csr_split_dense_head(A, fill, nullptr);
+}
+
+// The H update also produces H^T H (one pass over H instead of two) when the rank is 128 and
+// the factor is large enough for the pass to matter.  DNPEFF_FUSED_GRAM=0 switches it off.
+static bool fused_update(const dnpeff_nmf* h) {
+  if (const char* e = getenv("DNPEFF_FUSED_GRAM"))
+    if (atoi(e) == 0) return false;
+  return h->r == 128 && h->m >= 4096;
 }
 
 DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out) {
@@ -139,6 +151,8 @@ DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, d
           dmalloc(&h->H, mr) || dmalloc(&h->S, mr) || dmalloc(&h->G, (int64_t)rank * rank) ||
           dmalloc(&h->G2, (int64_t)rank * rank) || dmalloc(&h->gram_ws, ws) ||
           dmalloc(&h->dot_ws, DOT_BLOCKS + 2);
+  if (!s && fused_update(h))
+    s = dmalloc(&h->GH, (int64_t)rank * rank) || dmalloc(&h->gpart, xg_mu_gram_workspace_floats(h->m));
   if (!s) s = dnpeff_csr_sq_norm(A, &h->sq_norm_A);
   if (s) { dnpeff_nmf_destroy(h); return s; }
   *out = h;
@@ -148,6 +162,7 @@ DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, d
 DN_API int dnpeff_nmf_init_factors(dnpeff_nmf* nmf) {
   clear_error();
   DN_CHECK(nmf != nullptr, "handle is NULL");
+  nmf->gh_valid = false;
   DN_TRY(launch_init_uniform(0, nmf->n, nmf->r, nmf->seed, nmf->W));
   DN_TRY(launch_init_uniform(1, nmf->r, nmf->m, nmf->seed, nmf->H));
   return 0;
@@ -160,6 +175,7 @@ DN_API int dnpeff_nmf_set_factors(dnpeff_nmf* nmf, const float* W_nr, const floa
   if (W_nr)
     DN_HIP(hipMemcpy(nmf->W, W_nr, sizeof(float) * nmf->n * nmf->r, hipMemcpyHostToDevice));
   if (H_rm) {
+    nmf->gh_valid = false;
     DN_HIP(hipMemcpy(nmf->S, H_rm, sizeof(float) * nmf->m * nmf->r, hipMemcpyHostToDevice));
     DN_TRY(launch_transpose(nmf->r, nmf->m, nmf->S, nmf->H));
     DN_HIP(hipStreamSynchronize(stream()));
@@ -176,11 +192,15 @@ DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N_REDUCE));
   DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
   DN_TRY(h->prof.end());
-  DN_TRY(h->prof.begin(DNPEFF_K_GRAM_H));
-  DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
-  DN_TRY(h->prof.end());
+  const float* Gh = h->GH;
+  if (!h->gh_valid) {
+    DN_TRY(h->prof.begin(DNPEFF_K_GRAM_H));
+    DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
+    DN_TRY(h->prof.end());
+    Gh = h->G;
+  }
   DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_W));
-  DN_TRY(launch_xg_mu(h->n, h->r, h->W, h->G, h->Nw, h->eps, h->W2, nullptr));
+  DN_TRY(launch_xg_mu(h->n, h->r, h->W, Gh, h->Nw, h->eps, h->W2, nullptr));
   DN_TRY(h->prof.end());
   std::swap(h->W, h->W2);
   return 0;
@@ -196,7 +216,13 @@ DN_API int dnpeff_nmf_update_H(dnpeff_nmf* h) {
   DN_TRY(launch_gram(h->n, h->r, h->W, h->G, h->gram_ws));
   DN_TRY(h->prof.end());
   DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_H));
-  DN_TRY(launch_xg_mu(h->m, h->r, h->H, h->G, h->S, h->eps, h->S, nullptr));
+  if (h->GH && ((uintptr_t)h->H % 16) == 0) {
+    DN_TRY(launch_xg_mu_gram(h->m, h->H, h->G, h->S, h->eps, h->S, h->GH, h->gpart, h->G2, h->gram_ws));
+    h->gh_valid = true;
+  } else {
+    DN_TRY(launch_xg_mu(h->m, h->r, h->H, h->G, h->S, h->eps, h->S, nullptr));
+    h->gh_valid = false;
+  }
   DN_TRY(h->prof.end());
   std::swap(h->H, h->S);
   return 0;

@@ -896,6 +896,257 @@ static int launch_xg_mu_nb(int64_t rows, int r, const float* X, const float* G, 
 #undef DN_XG
 }
 
+// ---------------------------------------------------------------------------
+// The same update for r = 128 that also accumulates the Gram matrix of its OUTPUT, so that the
+// next A-side update does not have to read the new factor again: out = X * num / (X G + eps),
+// Gout += out^T out.
+//
+// After the epilogue a lane holds out[row(v, half)][32 cb + l32] in register v, where rows
+// row(v, 0) and row(v, 1) differ by 4: exactly the operand shape of v_mfma_f32_32x32x2f32 with
+// the row pair as contraction index.  The diagonal block (cb, cb) of the Gram matrix therefore
+// takes both operands from the registers; for the other blocks of the wave (cb, cb + 1 mod 4 and,
+// for waves 0 and 1, cb + 2) the second operand is read from the LDS tile, where every wave has
+// replaced X by its part of out (after a barrier: the other waves read X until their MFMAs and
+// epilogue are done).  10 distinct blocks in all; the reduction kernel mirrors
+// them.  The Gram accumulators are flushed every XGG_FLUSH tiles so that no fp32 sum runs over
+// more than 32,768 rows; the partial sums are added in fp64 in a fixed order.
+// ---------------------------------------------------------------------------
+constexpr int XGG_FLUSH = 512;
+constexpr int XGG_BLOCKS = 12;  // 4 waves x 3 block slots (the third is used by waves 0 and 1)
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_xg_mu_gram(const float* __restrict__ X, const float* __restrict__ G, const float* num,
+                 float eps, int64_t n_tiles, int n_flush, float* out, float* __restrict__ gpart) {
+  using C = XgReg<4>;
+  constexpr int r = C::R;
+  extern __shared__ __align__(16) float xl[];  // 2 slots of ROWS x LD
+  const int cb = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int col = 32 * cb + l32;
+
+  float g[C::KG][4];
+#pragma unroll
+  for (int kg = 0; kg < C::KG; kg++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) g[kg][s] = G[(8 * kg + 4 * half + s) * r + col];
+
+  const int lc = threadIdx.x % C::C4, lr = threadIdx.x / C::C4;
+  float4 R[C::NV];
+  auto fetch = [&](int64_t tile) {
+    const float* src = X + (tile * C::ROWS + lr) * (int64_t)r + 4 * lc;
+#pragma unroll
+    for (int q = 0; q < C::NV; q++)
+      R[q] = tile < n_tiles ? *reinterpret_cast<const float4*>(src + q * C::RSTEP * r)
+                            : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  };
+  auto commit = [&](float* slot) {
+#pragma unroll
+    for (int q = 0; q < C::NV; q++)
+      *reinterpret_cast<float4*>(slot + (lr + q * C::RSTEP) * C::LD + 4 * lc) = R[q];
+  };
+
+  acc16 ga[3];
+  auto ga_clear = [&]() {
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) ga[k][v] = 0.0f;
+  };
+  auto ga_flush = [&](int chunk) {
+    float* dst = gpart + (((int64_t)blockIdx.x * n_flush + chunk) * XGG_BLOCKS + 3 * cb) * 1024 + lane;
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) dst[k * 1024 + v * 64] = ga[k][v];
+  };
+  ga_clear();
+
+  int64_t tile = blockIdx.x;
+  fetch(tile);
+  commit(xl);
+  fetch(tile + gridDim.x);
+  __syncthreads();
+
+  const int lrow0 = 4 * half;
+  const unsigned off0 = (unsigned)(lrow0 * r + col);
+  const int cb1 = (cb + 1) & 3, cb2 = (cb + 2) & 3;
+  int it = 0;
+  for (; tile < n_tiles; it++, tile += gridDim.x) {
+    float* slot = xl + (it & 1) * C::SLOT;
+    const int64_t t0 = tile * C::ROWS * (int64_t)r;
+    const float* tnum = num + t0;
+    float* tout = out + t0;
+    float pn[C::RB][16];
+#pragma unroll
+    for (int b = 0; b < C::RB; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        pn[b][v] = (tnum + (32 * b + 8 * (v >> 2) + (v & 3)) * r)[off0];
+    acc16 acc[C::RB];
+#pragma unroll
+    for (int b = 0; b < C::RB; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[b][v] = 0.0f;
+
+    const float* arow = slot + l32 * C::LD + 4 * half;
+#pragma unroll
+    for (int kg = 0; kg < C::KG; kg++) {
+      float4 a[C::RB];
+#pragma unroll
+      for (int b = 0; b < C::RB; b++)
+        a[b] = *reinterpret_cast<const float4*>(arow + 32 * b * C::LD + 8 * kg);
+#pragma unroll
+      for (int b = 0; b < C::RB; b++) {
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].x, g[kg][0], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].y, g[kg][1], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].z, g[kg][2], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b].w, g[kg][3], acc[b], 0, 0, 0);
+      }
+    }
+
+    // the next tile goes to the other slot now (it was last read before the previous barrier),
+    // which frees its registers for the rest of the iteration
+    commit(xl + ((it + 1) & 1) * C::SLOT);
+
+    // epilogue: the result replaces the numerator registers
+#pragma unroll
+    for (int b = 0; b < C::RB; b++) {
+      float x[16];
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        x[v] = slot[(lrow0 + 32 * b + 8 * (v >> 2) + (v & 3)) * C::LD + col];
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int below = 32 * b + 8 * (v >> 2) + (v & 3);
+        const float q = pn[b][v] / (acc[b][v] + eps);
+        const float o = x[v] * q;
+        pn[b][v] = o;
+        (tout + below * r)[off0] = o;
+      }
+    }
+    __syncthreads();  // every wave is done with the X values of this slot
+#pragma unroll
+    for (int b = 0; b < C::RB; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        slot[(lrow0 + 32 * b + 8 * (v >> 2) + (v & 3)) * C::LD + col] = pn[b][v];
+    __syncthreads();
+
+    // Gram blocks of the new tile; the block pairs two apart, (0, 2) and (1, 3), are taken by
+    // waves 0 and 1 on even iterations and, transposed, by waves 2 and 3 on odd ones, so that
+    // all four SIMDs carry the same number of MFMAs
+    const bool third = (cb < 2) == ((it & 1) == 0);
+#pragma unroll
+    for (int b = 0; b < C::RB; b++) {
+      float y1[16], y2[16];
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int lrow = lrow0 + 32 * b + 8 * (v >> 2) + (v & 3);
+        y1[v] = slot[lrow * C::LD + 32 * cb1 + l32];
+        y2[v] = slot[lrow * C::LD + 32 * cb2 + l32];
+      }
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        ga[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(pn[b][v], pn[b][v], ga[0], 0, 0, 0);
+        ga[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(pn[b][v], y1[v], ga[1], 0, 0, 0);
+        if (third) ga[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(pn[b][v], y2[v], ga[2], 0, 0, 0);
+      }
+    }
+    if ((it + 1) % XGG_FLUSH == 0) {
+      ga_flush(it / XGG_FLUSH);
+      ga_clear();
+    }
+
+    fetch(tile + 2 * (int64_t)gridDim.x);
+    __syncthreads();
+  }
+  // the chunk in progress, then zeros for the chunks this workgroup never reached
+  int chunk = it / XGG_FLUSH;
+  if (it % XGG_FLUSH != 0 || it == 0) ga_flush(chunk++);
+  ga_clear();
+  for (; chunk < n_flush; chunk++) ga_flush(chunk);
+}
+
+// Gout[a][b] = sum of the partial blocks (fp64, fixed order), both triangles.  One thread per
+// element of the upper block triangle.  Block slot (w, k) holds the block (w, w + k mod 4);
+// element (i, j) of a block sits at register v = 4 (i / 8) + i % 4 of lane j + 32 ((i / 4) % 2).
+__global__ void __launch_bounds__(256)
+    k_xg_gram_reduce(const float* __restrict__ gpart, int64_t n_parts, float* __restrict__ Gout) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= 128 * 128) return;
+  const int a = e >> 7, b = e & 127;
+  const int ca = a >> 5, cbk = b >> 5, i = a & 31, j = b & 31;
+  if (ca > cbk) return;
+  auto at = [](int w, int k, int ii, int jj) {
+    return (3 * w + k) * 1024 + (4 * (ii >> 3) + (ii & 3)) * 64 + jj + 32 * ((ii >> 2) & 1);
+  };
+  int src0, src1 = -1;
+  switch (cbk - ca) {
+    case 0: src0 = at(ca, 0, i, j); break;
+    case 1: src0 = at(ca, 1, i, j); break;
+    case 2: src0 = at(ca, 2, i, j); src1 = at(cbk, 2, j, i); break;
+    default: src0 = at(3, 1, j, i); break;  // (0, 3) is held as (3, 0)
+  }
+  double s = 0.0;
+#pragma unroll 8
+  for (int64_t p = 0; p < n_parts; p++) s += (double)gpart[p * (XGG_BLOCKS * 1024) + src0];
+  if (src1 >= 0) {
+#pragma unroll 8
+    for (int64_t p = 0; p < n_parts; p++) s += (double)gpart[p * (XGG_BLOCKS * 1024) + src1];
+  }
+  Gout[a * 128 + b] = (float)s;
+  Gout[b * 128 + a] = (float)s;
+}
+
+// Workspace of the fused update in floats, for `rows` rows.
+int64_t xg_mu_gram_workspace_floats(int64_t rows) {
+  const int64_t tiles = rows / XgReg<4>::ROWS;
+  int64_t wgs = (int64_t)n_cus() * 2;
+  if (wgs > tiles) wgs = tiles > 0 ? tiles : 1;
+  const int64_t n_flush = ceil_div(ceil_div(tiles > 0 ? tiles : 1, wgs), XGG_FLUSH);
+  return wgs * n_flush * XGG_BLOCKS * 1024;
+}
+
+// out = X * num / (X G + eps) and Gout = out^T out for r = 128; rows >= 64.  The rows past the
+// last whole tile go through the plain kernels and their Gram matrix (workspace `gram_ws`, at
+// least gram_workspace_floats(64, 128) floats; `G_tmp` r x r) is added.
+__global__ void __launch_bounds__(256) k_add_inplace(float* __restrict__ a, const float* __restrict__ b, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) a[i] += b[i];
+}
+
+int launch_xg_mu_gram(int64_t rows, const float* X, const float* G, const float* num, float eps,
+                      float* out, float* Gout, float* gpart, float* G_tmp, float* gram_ws) {
+  using C = XgReg<4>;
+  constexpr int r = 128;
+  const size_t lds = sizeof(float) * 2 * C::SLOT;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_gram, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)lds));
+    attr_set = true;
+  }
+  const int64_t tiles = rows / C::ROWS;
+  DN_CHECK(tiles >= 1, "fused update needs at least one whole tile");
+  int64_t wgs = (int64_t)n_cus() * 2;
+  if (wgs > tiles) wgs = tiles;
+  const int64_t n_flush = ceil_div(ceil_div(tiles, wgs), XGG_FLUSH);
+  hipLaunchKernelGGL(k_xg_mu_gram, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps, tiles,
+                     (int)n_flush, out, gpart);
+  hipLaunchKernelGGL(k_xg_gram_reduce, dim3(128 * 128 / 256), dim3(256), 0, stream(), gpart,
+                     wgs * n_flush, Gout);
+  DN_LAUNCH_CHECK();
+  const int64_t head = tiles * C::ROWS;
+  if (head < rows) {
+    const int64_t off = head * r;
+    DN_TRY(launch_xg_mu_nb<4>(rows - head, r, X + off, G, num + off, eps, out + off, nullptr));
+    DN_TRY(launch_gram(rows - head, r, out + off, G_tmp, gram_ws));
+    hipLaunchKernelGGL(k_add_inplace, dim3(r * r / 256), dim3(256), 0, stream(), Gout, G_tmp, r * r);
+    DN_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
 int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const float* num, float eps,
                  float* out, float* D_out) {
   DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);

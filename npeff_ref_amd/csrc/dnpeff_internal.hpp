@@ -91,6 +91,10 @@ int64_t gram_tiles_workspace_floats(int64_t rows, int r);
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace);
 int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const float* num, float eps,
                  float* out, float* D_out);
+// r = 128: the update and the Gram matrix of its output in one pass (dense.hip).
+int64_t xg_mu_gram_workspace_floats(int64_t rows);
+int launch_xg_mu_gram(int64_t rows, const float* X, const float* G, const float* num, float eps,
+                      float* out, float* Gout, float* gpart, float* G_tmp, float* gram_ws);
 // dot with fp64 accumulation; result lands in *out_dev (one double, device).
 // partials: workspace of DOT_BLOCKS doubles.
 constexpr int DOT_BLOCKS = 2048;

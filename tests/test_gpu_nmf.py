@@ -244,3 +244,22 @@ def test_fit_after_nmf_on_the_same_matrix():
     assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
     A.close()
     B.close()
+
+
+def test_fused_gram_in_H_update_matches_the_two_pass_path(monkeypatch):
+    """r = 128: the H update accumulates H^T H of its own output, the W update uses it; rows past
+    the last 64-row tile go through the plain kernels and are added.  Same bar against the oracle
+    with the fusion switched off, and the two runs agree far inside it."""
+    args = (300, 40000, 2048, 128, 1e-8, 50)
+    nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(*args, seed=5)
+    assert A.n_cols % 64 != 0  # exercises the tail rows
+    assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
+    nmf.close()
+    A.close()
+    monkeypatch.setenv("DNPEFF_FUSED_GRAM", "0")
+    nmf2, A2, _, (W2, H2), _, hist2, _ = _run_case(*args, seed=5)
+    assert _nrm(W2, W64) < REL and _nrm(H2, H64) < REL
+    assert _nrm(W, W2.astype(np.float64)) < 1e-5 and _nrm(H, H2.astype(np.float64)) < 1e-5
+    assert abs(hist[-1][1] - hist2[-1][1]) / hist2[-1][1] < 1e-6
+    nmf2.close()
+    A2.close()
