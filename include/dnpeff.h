@@ -310,6 +310,15 @@ int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 int dnpeff_op_threshold_compact(int64_t count, const float* x, float divisor, float threshold,
                                 int32_t* idx_out, float* val_out, int64_t* n_kept);
 
+/* Per-example top-k of dense rows x[n_rows, count] (device): vals_out / idx_out [n_rows, k] get
+ * the k largest entries of each row in descending order, equal values in ascending index
+ * order, norms_out [n_rows] (may be NULL) the L2 norm of the whole row (sum of squares in
+ * fp64).  All buffers are device memory.  Replaces tf.math.top_k and the einsum norm in the
+ * PEF producer (npeff/fishers/d_pefs_computer.py:126-129 and :48-50); the outputs are the
+ * data/fisher/values, data/fisher/indices and data/dense_fisher_norms rows of the PEF file. */
+int dnpeff_topk_rows(int64_t n_rows, int64_t count, int64_t k, const float* x, float* vals_out,
+                     int32_t* idx_out, float* norms_out);
+
 /* G[r, r] = X^T X for X [rows, r].  cublasSgemm at device_contexts1.h:303,322. */
 int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr);
 

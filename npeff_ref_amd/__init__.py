@@ -30,6 +30,7 @@ from .binding import (  # noqa: F401
     op_mu,
     op_spmm_n,
     op_threshold_compact,
+    topk_rows,
     op_spmm_t,
     op_gram,
     op_xg_mu,

@@ -60,6 +60,7 @@ SIGNATURES = {
     "dnpeff_csr_kept_indices": (C.c_int, [_p, _p]),
     "dnpeff_csr_sq_norm": (C.c_int, [_p, C.POINTER(_f64)]),
     "dnpeff_csr_build_transpose": (C.c_int, [_p]),
+    "dnpeff_topk_rows": (C.c_int, [C.c_int64, C.c_int64, C.c_int64, _p, _p, _p, _p]),
     "dnpeff_op_threshold_compact": (C.c_int, [C.c_int64, _p, C.c_float, C.c_float, _p, _p, C.POINTER(C.c_int64)]),
     "dnpeff_csr_split_dense_head": (C.c_int, [_p, C.c_double, C.POINTER(C.c_int64)]),
     "dnpeff_csr_head_info": (C.c_int, [_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
@@ -240,6 +241,17 @@ def op_spsp_dense(A: "Csr", B: "Csr", out: DeviceArray):
 
 def op_init_uniform(matrix_id: int, logical_rows: int, logical_cols: int, seed: int, x: DeviceArray):
     _check(lib.dnpeff_op_init_uniform(matrix_id, logical_rows, logical_cols, seed & 0xFFFFFFFFFFFFFFFF, x.ptr))
+
+
+def topk_rows(x: "DeviceArray", k: int):
+    """(values [n, k], indices [n, k], norms [n]) of the k largest entries of each row of x."""
+    n, count = x.shape
+    vals = DeviceArray((n, k), dtype=np.float32)
+    idx = DeviceArray((n, k), dtype=np.int32)
+    norms = DeviceArray((n,), dtype=np.float32)
+    _check(lib.dnpeff_topk_rows(n, count, k, x.ptr, vals.ptr, idx.ptr, norms.ptr))
+    sync()
+    return vals.numpy(), idx.numpy(), norms.numpy()
 
 
 def op_threshold_compact(x: "DeviceArray", divisor: float, threshold: float):

@@ -15,6 +15,8 @@ import os
 import sys
 import time
 
+import numpy as np
+
 sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
 import npeff_ref_amd as d  # noqa: E402
@@ -22,7 +24,7 @@ import npeff_ref_amd as d  # noqa: E402
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--op", required=True, choices=["mu", "gram", "xg_mu", "copy", "spmm_n", "spmm_t"])
+    ap.add_argument("--op", required=True, choices=["mu", "gram", "xg_mu", "copy", "spmm_n", "spmm_t", "topk"])
     ap.add_argument("--rows", type=int, default=4_000_000)
     ap.add_argument("--rank", type=int, default=128)
     ap.add_argument("--iters", type=int, default=5)
@@ -50,6 +52,15 @@ def main():
         fn = (lambda: d.op_spmm_n(A, r, H, N)) if a.op == "spmm_n" else (lambda: d.op_spmm_t(A, r, W, T))
         work = 8 * z + 4 * (n + 1 if a.op == "spmm_n" else m + 1) + 4 * r * m + 4 * n * r
         desc = f"n={n} m={m} nnz={z} r={r}"
+    elif a.op == "topk":
+        # --rows examples of --m-full dense Fisher values each, the --k largest kept
+        rows, count, k = a.rows, a.m_full, a.k
+        X = uniform(rows, count, 2)
+        vals, idx = d.DeviceArray((rows, k)), d.DeviceArray((rows, k), dtype=np.int32)
+        norms = d.DeviceArray((rows,))
+        fn = lambda: d.binding._check(d.lib.dnpeff_topk_rows(rows, count, k, X.ptr, vals.ptr, idx.ptr, norms.ptr))
+        work = 4 * rows * count
+        desc = f"rows={rows} count={count} k={k}"
     else:
         rows = a.rows
         X = uniform(rows, r, 2)

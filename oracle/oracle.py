@@ -284,6 +284,17 @@ def sparsify_H(W, H_rm, threshold):
             np.concatenate(cols).astype(np.int32))
 
 
+def topk_rows(x, k):
+    """Per row: the k largest entries in descending order, equal values by ascending index
+    (tf.math.top_k's rule), and the L2 norm of the whole row.
+    npeff/fishers/d_pefs_computer.py:126-129, :48-50."""
+    x = np.asarray(x, dtype=np.float32)
+    order = np.argsort(-x.astype(np.float64), axis=1, kind="stable")[:, :k]
+    vals = np.take_along_axis(x, order, axis=1)
+    norms = np.sqrt(np.sum(x.astype(np.float64) ** 2, axis=1)).astype(np.float32)
+    return vals, order.astype(np.int32), norms
+
+
 def have_ref():
     return _ref is not None
 

@@ -303,3 +303,24 @@ def test_threshold_compact_bit_exact(n, div, thr):
     keep = q >= np.float32(thr)
     assert np.array_equal(idx, np.nonzero(keep)[0].astype(np.int32))
     assert np.array_equal(val, q[keep])
+
+
+@pytest.mark.parametrize("n,count,k", [(3, 100000, 4096), (2, 5000, 1), (1, 70001, 70001), (4, 30000, 5000),
+                                       (1, 3_000_000, 65536)])
+@pytest.mark.parametrize("cap", [None, 0, 9000])
+def test_topk_rows_bit_exact(n, count, k, cap, monkeypatch):
+    """Device top-k sparsifier vs the full-sort restatement: same values, same indices (ties by
+    ascending index), zeros and repeated values included; both the two-read path and the
+    exact-threshold path for crowded bins (forced with a zero cap)."""
+    if cap is not None:
+        monkeypatch.setenv("DNPEFF_TOPK_FAST_CAP", str(cap))
+    rng = np.random.default_rng(count + k)
+    x = rng.lognormal(-8, 2, size=(n, count)).astype(np.float32)
+    x[0, ::5] = 0.0
+    x[-1, 1::3] = np.float32(0.125)  # far more ties than k when k is small
+    if count > 1000:
+        x[0, 17] = np.float32(-1.0)  # a negative entry sorts below the zeros
+    v, i, nrm = d.topk_rows(d.DeviceArray.from_numpy(x), k)
+    wv, wi, wn = orc.topk_rows(x, k)
+    assert np.array_equal(v, wv) and np.array_equal(i, wi)
+    assert np.all(np.abs(nrm - wn) <= 1e-6 * wn)

@@ -163,3 +163,25 @@ def test_sparsify_H_keeps_the_product_and_thresholds_unit_norm_rows():
         dense[k, c] = vals[offs[k]:offs[k + 1]]
     assert np.array_equal(dense, np.where(Hn >= np.float32(thr), Hn, 0).astype(np.float32))
     assert np.array_equal(W3, W2)
+
+
+def test_topk_rows_against_a_full_sort_and_known_cases():
+    """Known answer with ties (lower index first), and the defining property on random rows:
+    the kept values are the k largest of a full sort, every dropped entry is <= the smallest
+    kept one, and the indices point at the values."""
+    x = np.array([[1.0, 5.0, 5.0, 0.0, 7.0, 5.0]], dtype=np.float32)
+    v, i, nrm = orc.topk_rows(x, 4)
+    assert v.tolist() == [[7.0, 5.0, 5.0, 5.0]] and i.tolist() == [[4, 1, 2, 5]]
+    assert np.isclose(nrm[0], np.sqrt(1 + 75 + 49))
+    rng = np.random.default_rng(2)
+    x = rng.lognormal(-8, 2, size=(3, 5000)).astype(np.float32)
+    x[1, ::7] = 0.25  # many ties
+    k = 700
+    v, i, _ = orc.topk_rows(x, k)
+    for r in range(3):
+        assert np.array_equal(v[r], np.sort(x[r])[::-1][:k])
+        assert np.array_equal(x[r, i[r]], v[r]) and len(set(i[r].tolist())) == k
+        rest = np.delete(x[r], i[r])
+        assert rest.max() <= v[r, -1]
+        same = np.flatnonzero(np.diff(v[r]) == 0)
+        assert np.all(i[r, same] < i[r, same + 1])
