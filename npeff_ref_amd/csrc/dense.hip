@@ -1072,30 +1072,40 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 // element (i, j) of a block sits at register v = 4 (i / 8) + i % 4 of lane j + 32 ((i / 4) % 2).
 __global__ void __launch_bounds__(256)
     k_xg_gram_reduce(const float* __restrict__ gpart, int64_t n_parts, float* __restrict__ Gout) {
-  const int e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= 128 * 128) return;
+  // 32 elements per workgroup, 8 threads per element: thread q sums the parts q, q + 8, ...,
+  // the eight sums are added in order
+  __shared__ double red[8][32];
+  const int q = threadIdx.x >> 5;
+  const int e = blockIdx.x * 32 + (threadIdx.x & 31);
   const int a = e >> 7, b = e & 127;
   const int ca = a >> 5, cbk = b >> 5, i = a & 31, j = b & 31;
-  if (ca > cbk) return;
   auto at = [](int w, int k, int ii, int jj) {
     return (3 * w + k) * 1024 + (4 * (ii >> 3) + (ii & 3)) * 64 + jj + 32 * ((ii >> 2) & 1);
   };
-  int src0, src1 = -1;
-  switch (cbk - ca) {
-    case 0: src0 = at(ca, 0, i, j); break;
-    case 1: src0 = at(ca, 1, i, j); break;
-    case 2: src0 = at(ca, 2, i, j); src1 = at(cbk, 2, j, i); break;
-    default: src0 = at(3, 1, j, i); break;  // (0, 3) is held as (3, 0)
-  }
   double s = 0.0;
+  if (ca <= cbk) {
+    int src0, src1 = -1;
+    switch (cbk - ca) {
+      case 0: src0 = at(ca, 0, i, j); break;
+      case 1: src0 = at(ca, 1, i, j); break;
+      case 2: src0 = at(ca, 2, i, j); src1 = at(cbk, 2, j, i); break;
+      default: src0 = at(3, 1, j, i); break;  // (0, 3) is held as (3, 0)
+    }
 #pragma unroll 8
-  for (int64_t p = 0; p < n_parts; p++) s += (double)gpart[p * (XGG_BLOCKS * 1024) + src0];
-  if (src1 >= 0) {
+    for (int64_t p = q; p < n_parts; p += 8) s += (double)gpart[p * (XGG_BLOCKS * 1024) + src0];
+    if (src1 >= 0) {
 #pragma unroll 8
-    for (int64_t p = 0; p < n_parts; p++) s += (double)gpart[p * (XGG_BLOCKS * 1024) + src1];
+      for (int64_t p = q; p < n_parts; p += 8) s += (double)gpart[p * (XGG_BLOCKS * 1024) + src1];
+    }
   }
-  Gout[a * 128 + b] = (float)s;
-  Gout[b * 128 + a] = (float)s;
+  red[q][threadIdx.x & 31] = s;
+  __syncthreads();
+  if (q == 0 && ca <= cbk) {
+    double t = 0.0;
+    for (int u = 0; u < 8; u++) t += red[u][threadIdx.x];
+    Gout[a * 128 + b] = (float)t;
+    Gout[b * 128 + a] = (float)t;
+  }
 }
 
 // Workspace of the fused update in floats, for `rows` rows.
@@ -1133,7 +1143,7 @@ int launch_xg_mu_gram(int64_t rows, const float* X, const float* G, const float*
   const int64_t n_flush = ceil_div(ceil_div(tiles, wgs), XGG_FLUSH);
   hipLaunchKernelGGL(k_xg_mu_gram, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps, tiles,
                      (int)n_flush, out, gpart);
-  hipLaunchKernelGGL(k_xg_gram_reduce, dim3(128 * 128 / 256), dim3(256), 0, stream(), gpart,
+  hipLaunchKernelGGL(k_xg_gram_reduce, dim3(128 * 128 / 32), dim3(256), 0, stream(), gpart,
                      wgs * n_flush, Gout);
   DN_LAUNCH_CHECK();
   const int64_t head = tiles * C::ROWS;
