@@ -61,13 +61,14 @@ def algorithmic(cls, n, m, z, r, fused_gram=False):
         return "hbm", 8 * n * r
     if cls == "spmm_t":
         return "hbm", 8 * z + P * (m + 1) + 4 * n * r + 4 * r * m
+    # a Gram matrix is symmetric: r (r + 1) / 2 distinct dot products of length e
     if cls == "gram_H":
-        return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 4 * m * r + 4 * r * r)
+        return ("mfma", m * r * (r + 1)) if r >= 64 else ("hbm", 4 * m * r + 4 * r * r)
     if cls == "gram_W":
-        return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 4 * n * r + 4 * r * r)
+        return ("mfma", n * r * (r + 1)) if r >= 64 else ("hbm", 4 * n * r + 4 * r * r)
     if cls == "xg_mu_H":
         if fused_gram:
-            return "mfma", 4 * m * r * r
+            return "mfma", 2 * m * r * r + m * r * (r + 1)
         return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 12 * m * r + 4 * r * r)
     if cls == "xg_mu_W":
         return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 12 * n * r + 4 * r * r)

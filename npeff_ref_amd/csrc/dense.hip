@@ -715,8 +715,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
-  const int64_t tile = blockIdx.x / n_chunks;
-  const int n0 = (int)(blockIdx.x % n_chunks) * 128;
+  // Workgroups are dealt to the 8 XCDs round-robin by their number; the column chunks of one row
+  // tile are numbered 8 apart so that they share an XCD, i.e. an L2, and X comes in once.
+  const int64_t grp = blockIdx.x / (8 * n_chunks);
+  const int rem = (int)(blockIdx.x % (8 * n_chunks));
+  const int64_t tile = grp * 8 + rem % 8;
+  if (tile * 128 >= rows) return;
+  const int n0 = (rem / 8) * 128;
   const int64_t row0 = tile * 128;
   const int n_kt = r / XGT_KB;
 
@@ -844,7 +849,7 @@ static int launch_xg_mu_tile(int64_t rows, int r, const float* X, const float* G
     attr_set = true;
   }
   const int n_chunks = r / 128;
-  const int64_t wgs = ceil_div(rows, 128) * n_chunks;
+  const int64_t wgs = ceil_div(ceil_div(rows, 128), 8) * 8 * n_chunks;
   DN_CHECK(wgs < ((int64_t)1 << 24), "xg_mu: too many tiles for one launch");
   const dim3 grid((unsigned)wgs), block(256);
   if (D_out)

@@ -43,12 +43,26 @@ __global__ void __launch_bounds__(256)
           int64_t M, int64_t M_pad, int upper_only,
           float* __restrict__ out) {
   extern __shared__ __align__(16) float lds[];  // 2 * PTQ_SLOT floats
-  if (upper_only && blockIdx.x > blockIdx.y) return;  // symmetric product: tiles (i <= j) only
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
-  const int64_t m0 = (int64_t)blockIdx.x * 128;
-  const int n0 = blockIdx.y * 128;
+  // Symmetric product (upper_only = number of 128-wide tiles per side): grid.x numbers the tile
+  // pairs (i <= j) row by row.  Every workgroup of the grid works: the hardware deals workgroups
+  // to the XCDs round-robin by their linear number, and a grid with idle numbers at a fixed
+  // stride would leave whole XCDs without work.
+  int ti = blockIdx.x, tj = blockIdx.y;
+  if (upper_only) {
+    int p = blockIdx.x, row_len = upper_only;
+    ti = 0;
+    while (p >= row_len) {
+      p -= row_len;
+      ti++;
+      row_len--;
+    }
+    tj = ti + p;
+  }
+  const int64_t m0 = (int64_t)ti * 128;
+  const int n0 = tj * 128;
   // the K tiles are dealt to the slices round-robin (slice z owns tiles z, z + S, ...), so that
   // at any moment the workgroups read one contiguous window of P and Q
   const int64_t all_tiles = (K + PTQ_KB - 1) / PTQ_KB;
@@ -180,6 +194,7 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
   DN_CHECK(M_pad % 128 == 0 && ldp % 4 == 0 && r % 4 == 0, "dense product: misaligned operands");
   DN_CHECK(M_pad / 128 < ((int64_t)1 << 22), "dense product: too many row tiles");
   dim3 grid((unsigned)(M_pad / 128), (unsigned)ceil_div(r, 128), (unsigned)slices);
+  if (upper_only) grid = dim3((unsigned)(upper_only * (upper_only + 1) / 2), 1, (unsigned)slices);
   hipLaunchKernelGGL(k_ptq, grid, dim3(256), lds, stream(), P, ldp, K, Q, r, M, M_pad,
                      upper_only, out);
   DN_LAUNCH_CHECK();
@@ -219,7 +234,7 @@ __global__ void __launch_bounds__(256)
 
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace) {
   const int64_t slices = gram_tiles_slices(rows, r);
-  DN_TRY(launch_ptq(X, r, rows, X, r, r, r, slices, workspace, 1));
+  DN_TRY(launch_ptq(X, r, rows, X, r, r, r, slices, workspace, r / 128));
   hipLaunchKernelGGL(k_gram_tiles_reduce, dim3((unsigned)ceil_div((int64_t)r * r, 256)), dim3(256), 0,
                      stream(), workspace, slices, r, G);
   DN_LAUNCH_CHECK();
