@@ -329,24 +329,51 @@ __global__ void __launch_bounds__(256)
   const int64_t cp = lane <= SPMM_T_COLS ? colptr[jc] : 0;
   const int cp_lo = (int)(uint32_t)(cp & 0xffffffffLL), cp_hi = (int)(cp >> 32);
 
-  for (int round = 0; round * G < SPMM_T_COLS; round++) {
+  // The (row, value) pairs of a round's columns are requested one round ahead, so that their
+  // latency overlaps the gathers of the round before: two dependent memory round trips per
+  // column would otherwise bound the kernel.
+  auto request = [&](int round, int64_t& p0, int& len, bool& active, int& e_i, float& e_v) {
     const int jl = round * G + grp;
     const int64_t j = j0 + jl;
-    const int64_t p0 = ((int64_t)__shfl(cp_hi, jl) << 32) | (uint32_t)__shfl(cp_lo, jl);
-    const int64_t p1 = ((int64_t)__shfl(cp_hi, jl + 1) << 32) | (uint32_t)__shfl(cp_lo, jl + 1);
-    const bool active = j < m && (p1 - p0) <= SPMM_T_LONG;  // longer ones: k_spmm_t_long
-    const int len = active ? (int)(p1 - p0) : 0;
+    p0 = ((int64_t)__shfl(cp_hi, jl & 63) << 32) | (uint32_t)__shfl(cp_lo, jl & 63);
+    const int64_t p1 =
+        ((int64_t)__shfl(cp_hi, (jl + 1) & 63) << 32) | (uint32_t)__shfl(cp_lo, (jl + 1) & 63);
+    active = jl < SPMM_T_COLS && j < m && (p1 - p0) <= SPMM_T_LONG;  // longer: k_spmm_t_long
+    len = active ? (int)(p1 - p0) : 0;
+    e_i = 0;
+    e_v = 0.0f;
+    if (sub < len) {
+      e_i = rowind[p0 + sub];
+      e_v = tvals[p0 + sub];
+    }
+  };
+  int64_t nx_p0;
+  int nx_len, nx_i;
+  bool nx_active;
+  float nx_v;
+  request(0, nx_p0, nx_len, nx_active, nx_i, nx_v);
+
+  for (int round = 0; round * G < SPMM_T_COLS; round++) {
+    const int64_t j = j0 + round * G + grp;
+    const int64_t p0 = nx_p0;
+    const int len = nx_len;
+    const bool active = nx_active;
+    int my_i = nx_i;
+    float my_v = nx_v;
+    request(round + 1, nx_p0, nx_len, nx_active, nx_i, nx_v);
     float4 acc[T];
 #pragma unroll
     for (int t = 0; t < T; t++) acc[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
     for (int base = 0; __any(base < len); base += LPR) {
-      const int e = base + sub;
-      int my_i = 0;
-      float my_v = 0.0f;
-      if (e < len) {
-        my_i = rowind[p0 + e];
-        my_v = tvals[p0 + e];
+      if (base > 0) {  // columns longer than a lane group: further batches are loaded here
+        const int e = base + sub;
+        my_i = 0;
+        my_v = 0.0f;
+        if (e < len) {
+          my_i = rowind[p0 + e];
+          my_v = tvals[p0 + e];
+        }
       }
       const int cnt = len - base;  // entries of this group in the batch (may be <= 0 or > LPR)
       // the wave walks to the largest count among its groups
