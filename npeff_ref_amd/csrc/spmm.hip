@@ -30,6 +30,7 @@ struct GatherDword {
   float acc[VPL];
   bool ok[VPL];
   int lane;
+  bool small = false;  // (unused here) X smaller than 4 GB
 
   // `width` components starting at the pointers given to run() and store()
   __device__ inline void init(int lane_, int width) {
@@ -98,6 +99,7 @@ struct GatherVec4 {
   float4 acc[T];
   bool ok[T];
   int lane, sub, grp;
+  bool small = false;  // X smaller than 4 GB: 32-bit row offsets
 
   // `width` components starting at the pointers given to run() and store()
   __device__ inline void init(int lane_, int width) {
@@ -121,22 +123,24 @@ struct GatherVec4 {
         my_i = idx[p + lane];
         my_v = val[p + lane];
       }
+      // Lanes past the batch hold (row 0, value 0): a padded step gathers row 0 with weight 0,
+      // so the steps need no predicates.  Row offsets are 32-bit when X is smaller than 4 GB
+      // (one multiply-add per gathered row).
       const int nsteps = (cnt + G - 1) / G;
       for (int q = 0; q < nsteps; q += UNR) {
         float4 h[UNR][T];
         float a[UNR];
 #pragma unroll
         for (int uu = 0; uu < UNR; uu++) {
-          const int u = (q + uu) * G + grp;
-          const bool valid = u < cnt;
-          const int j = __shfl(my_i, u & 63);
-          a[uu] = __shfl(my_v, u & 63);
-          const float* x = X + (int64_t)j * r + 4 * sub;
+          const int u = ((q + uu) * G + grp) & 63;
+          const int j = __shfl(my_i, u);
+          a[uu] = __shfl(my_v, u);
+          const float* x = small ? X + ((unsigned)j * (unsigned)r + 4u * (unsigned)sub)
+                                 : X + (int64_t)j * r + 4 * sub;
 #pragma unroll
           for (int t = 0; t < T; t++)
-            h[uu][t] = (valid && ok[t]) ? *reinterpret_cast<const float4*>(x + 256 * t)
-                                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          if (!valid) a[uu] = 0.0f;
+            h[uu][t] = ok[t] ? *reinterpret_cast<const float4*>(x + 256 * t)
+                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int uu = 0; uu < UNR; uu++)
@@ -284,7 +288,7 @@ template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_short(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
                    const float* __restrict__ tvals, int64_t m, int r, int n_slices,
-                   const float* __restrict__ W, float* __restrict__ T) {
+                   const float* __restrict__ W, float* __restrict__ T, bool w_small) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int slice = blockIdx.x % n_slices, width = r / n_slices;
   // gridDim.x is a multiple of n_slices: the slice of a workgroup never changes
@@ -296,6 +300,7 @@ __global__ void __launch_bounds__(256)
     if (p1 - p0 > SPMM_T_LONG) continue;  // written by k_spmm_t_long
     GT g;
     g.init(lane, width);
+    g.small = w_small;
     g.run(rowind, tvals, p0, p1, W + slice * width, r);
     g.store(T + j * r + slice * width);
   }
@@ -313,7 +318,7 @@ template <int LPR, int T>
 __global__ void __launch_bounds__(256)
     k_spmm_t_grouped(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
                      const float* __restrict__ tvals, int64_t m, int r,
-                     const float* __restrict__ W, float* __restrict__ Tout) {
+                     const float* __restrict__ W, float* __restrict__ Tout, bool w_small) {
   constexpr int G = 64 / LPR;
   constexpr int UNR = T >= 4 ? 1 : T == 2 ? 2 : 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -322,7 +327,7 @@ __global__ void __launch_bounds__(256)
   if (j0 >= m) return;
   bool ok[T];
 #pragma unroll
-  for (int t = 0; t < T; t++) ok[t] = 4 * (sub + 64 * t) < r;
+  for (int t = 0; t < T; t++) ok[t] = 4 * (sub + LPR * t) < r;
 
   // colptr[j0 + lane] for lane <= SPMM_T_COLS, as two 32-bit halves for the shuffles
   const int64_t jc = j0 + lane < m ? j0 + lane : m;
@@ -384,21 +389,26 @@ __global__ void __launch_bounds__(256)
         cmax = c > cmax ? c : cmax;
       }
       if (cmax > LPR) cmax = LPR;
-      for (int u = 0; u < cmax; u += UNR) {
+      // Whole blocks of UNR entries with their loads in flight together, then the rest one by
+      // one: most columns hold one or two entries.  Lanes past a group's entries hold
+      // (row 0, value 0), so a step that a shorter group only accompanies gathers row 0 with
+      // weight 0 and needs no predicate; offsets into W are 32-bit when W is below 4 GB.
+      auto wrow = [&](int jrow) {
+        return w_small ? W + ((unsigned)jrow * (unsigned)r + 4u * (unsigned)sub)
+                       : W + (int64_t)jrow * r + 4 * sub;
+      };
+      int u = 0;
+      for (; u + UNR <= cmax; u += UNR) {
         float4 h[UNR][T];
         float a[UNR];
 #pragma unroll
         for (int uu = 0; uu < UNR; uu++) {
-          const int ue = u + uu;
-          const bool valid = ue < cnt && ue < LPR;
-          const int jrow = __shfl(my_i, gbase + (ue & (LPR - 1)));
-          a[uu] = __shfl(my_v, gbase + (ue & (LPR - 1)));
-          const float* x = W + (int64_t)jrow * r + 4 * sub;
+          const float* x = wrow(__shfl(my_i, gbase + u + uu));
+          a[uu] = __shfl(my_v, gbase + u + uu);
 #pragma unroll
           for (int t = 0; t < T; t++)
-            h[uu][t] = (valid && ok[t]) ? *reinterpret_cast<const float4*>(x + 256 * t)
-                                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          if (!valid) a[uu] = 0.0f;
+            h[uu][t] = ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
+                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int uu = 0; uu < UNR; uu++)
@@ -410,11 +420,24 @@ __global__ void __launch_bounds__(256)
             acc[t].w = fmaf(a[uu], h[uu][t].w, acc[t].w);
           }
       }
+      for (; u < cmax; u++) {
+        const float* x = wrow(__shfl(my_i, gbase + u));
+        const float a = __shfl(my_v, gbase + u);
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+          const float4 h = ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
+                                 : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          acc[t].x = fmaf(a, h.x, acc[t].x);
+          acc[t].y = fmaf(a, h.y, acc[t].y);
+          acc[t].z = fmaf(a, h.z, acc[t].z);
+          acc[t].w = fmaf(a, h.w, acc[t].w);
+        }
+      }
     }
     if (active) {
 #pragma unroll
       for (int t = 0; t < T; t++)
-        if (ok[t]) *reinterpret_cast<float4*>(Tout + j * r + 4 * (sub + 64 * t)) = acc[t];
+        if (ok[t]) *reinterpret_cast<float4*>(Tout + j * r + 4 * (sub + LPR * t)) = acc[t];
     }
   }
 }
@@ -423,7 +446,7 @@ template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_long(const int32_t* __restrict__ long_cols, const int64_t* __restrict__ colptr,
                   const int32_t* __restrict__ rowind, const float* __restrict__ tvals, int r,
-                  int n_slices, const float* __restrict__ W, float* __restrict__ T) {
+                  int n_slices, const float* __restrict__ W, float* __restrict__ T, bool w_small) {
   extern __shared__ __align__(16) float red_dyn[];  // [4][width]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int slice = blockIdx.x % n_slices, width = r / n_slices;
@@ -435,6 +458,7 @@ __global__ void __launch_bounds__(256)
   if (w1 > p1) w1 = p1;
   GT g;
   g.init(lane, width);
+  g.small = w_small;
   g.run(rowind, tvals, w0, w1, W + slice * width, r);
   g.store(red_dyn + wave * width);
   __syncthreads();
@@ -665,12 +689,13 @@ int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_m
   if (wgs > max_wgs) wgs = max_wgs;
   dim3 grid((unsigned)wgs), block(256);
   const bool grouped = aligned && r % 4 == 0 && n_slices == 1;
+  const bool w_small = (double)A->n_rows * r * 4.0 < 4.0e9;  // 32-bit offsets into W
   if (grouped) {
     dim3 gg((unsigned)ceil_div(A->n_cols, 4 * SPMM_T_COLS));
     const int r4 = r / 4;
 #define DN_GROUPED(LPR, T)                                                                     \
   hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T>), gg, block, 0, stream(), A->colptr, A->rowind, \
-                     A->tvals, A->n_cols, r, W_nr, T_mr)
+                     A->tvals, A->n_cols, r, W_nr, T_mr, w_small)
     if (r4 <= 4) DN_GROUPED(4, 1);
     else if (r4 <= 8) DN_GROUPED(8, 1);
     else if (r4 <= 16) DN_GROUPED(16, 1);
@@ -684,12 +709,12 @@ int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_m
     using GT = typename decltype(tag)::type;
     if (!grouped)
       hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), A->colptr, A->rowind,
-                         A->tvals, A->n_cols, r, n_slices, W_nr, T_mr);
+                         A->tvals, A->n_cols, r, n_slices, W_nr, T_mr, w_small);
     if (A->n_long > 0) {
       dim3 grid_l((unsigned)(A->n_long * n_slices));
       const size_t lds = sizeof(float) * 4 * (size_t)width;
       hipLaunchKernelGGL((k_spmm_t_long<GT>), grid_l, block, lds, stream(), A->long_cols,
-                         A->colptr, A->rowind, A->tvals, r, n_slices, W_nr, T_mr);
+                         A->colptr, A->rowind, A->tvals, r, n_slices, W_nr, T_mr, w_small);
     }
     return 0;
   });
