@@ -757,6 +757,30 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+  // element (i, j, v): row 64 wm + 32 i + 8 (v / 4) + 4 half + v % 4, column n0 + 64 wn + 32 j + l32
+  const int64_t t0 = (row0 + 64 * wm + 4 * half) * (int64_t)r + n0 + 64 * wn;
+  const float* tnum = num + t0;
+  const float* tx = X + t0;
+  float* tout = out + t0;
+  float* tD = WITH_D ? D_out + t0 : nullptr;
+  const int64_t rows_left = rows - (row0 + 64 * wm + 4 * half);  // rows at and below the lane's first
+  float pn[2][16], px[2][16];
+  auto request = [&](int blk, float (&n_)[16], float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int below = 32 * i + 8 * (v >> 2) + (v & 3);
+      // rows past the end are clamped to the lane's first row (never stored)
+      const int64_t off = (below < rows_left ? below : 0) * (int64_t)r + 32 * j + l32;
+      n_[v] = tnum[off];
+      x_[v] = tx[off];
+    }
+  };
+  // the epilogue operands of the first two blocks are requested before the contraction starts
+  if (rows_left > 0) {
+    request(0, pn[0], px[0]);
+    request(1, pn[1], px[1]);
+  }
   fetch(0);
   commit(tl);
   fetch(1);
@@ -786,31 +810,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, b[j][3], acc[i][j], 0, 0, 0);
         }
     }
-    // the other slot was last read before the previous barrier
-    commit(tl + ((kt + 1) & 1) * XGT_SLOT);
-    fetch(kt + 2);
-    __syncthreads();
+    if (kt + 1 < n_kt) {
+      // the other slot was last read before the previous barrier
+      commit(tl + ((kt + 1) & 1) * XGT_SLOT);
+      fetch(kt + 2);
+      __syncthreads();
+    }
   }
 
-  // element (i, j, v): row 64 wm + 32 i + 8 (v / 4) + 4 half + v % 4, column n0 + 64 wn + 32 j + l32
-  const int64_t t0 = (row0 + 64 * wm + 4 * half) * (int64_t)r + n0 + 64 * wn;
-  const float* tnum = num + t0;
-  const float* tx = X + t0;
-  float* tout = out + t0;
-  float* tD = WITH_D ? D_out + t0 : nullptr;
-  const int64_t rows_left = rows - (row0 + 64 * wm + 4 * half);  // rows at and below the lane's first
-  float pn[2][16], px[2][16];
-  auto request = [&](int blk, float (&n_)[16], float (&x_)[16]) {
-    const int i = blk >> 1, j = blk & 1;
-#pragma unroll
-    for (int v = 0; v < 16; v++) {
-      const int below = 32 * i + 8 * (v >> 2) + (v & 3);
-      // rows past the end are clamped to the lane's first row (never stored)
-      const int64_t off = (below < rows_left ? below : 0) * (int64_t)r + 32 * j + l32;
-      n_[v] = tnum[off];
-      x_[v] = tx[off];
-    }
-  };
   auto finish = [&](int blk, const float (&n_)[16], const float (&x_)[16]) {
     const int i = blk >> 1, j = blk & 1;
 #pragma unroll
@@ -826,8 +833,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
   };
   if (rows_left > 0) {
-    request(0, pn[0], px[0]);
-    request(1, pn[1], px[1]);
     finish(0, pn[0], px[0]);
     request(2, pn[0], px[0]);
     finish(1, pn[1], px[1]);
