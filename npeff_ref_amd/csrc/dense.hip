@@ -480,10 +480,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int64_t row = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        // element 0 stands in for the ones outside the matrix: unconditional loads, which the
+        // compiler can issue together (a branch per load would serialise them)
         const bool ok = cok[i] && row < rows;
         const int64_t idx = ok ? row * (int64_t)r + col : 0;
-        pn[i][v] = ok ? num[idx] : 0.0f;
-        px[i][v] = ok ? X[idx] : 0.0f;
+        pn[i][v] = num[idx];
+        px[i][v] = X[idx];
       }
     }
 
