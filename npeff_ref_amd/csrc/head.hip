@@ -11,7 +11,6 @@
 // the second.
 #include "dnpeff_internal.hpp"
 
-#include <type_traits>
 
 namespace dn {
 
@@ -20,8 +19,8 @@ typedef float acc16 __attribute__((ext_vector_type(16)));
 // ---------------------------------------------------------------------------
 // C[slice] = P[k in slice]^T Q[k in slice]
 //
-// A workgroup of 4 waves owns a 128 x 128 tile of C and a contiguous range of K, streamed in
-// tiles of 32 contraction rows through two LDS slots (P tile then Q tile, 16 KB each), fetched
+// A workgroup of 4 waves owns a 128 x 128 tile of C and one slice of K (every S-th tile of 32
+// contraction rows), streamed through two LDS slots (P tile then Q tile, 20 KB each), fetched
 // with 16-byte loads two tiles ahead into registers and written to LDS as they are (16-byte
 // stores).  v_mfma_f32_32x32x2f32 takes from lane l A[i = l%32][k = l/32] and
 // B[k = l/32][j = l%32]: a lane reads P[k][32 a + i] and Q[k][32 b + j] of its blocks with 4-byte
