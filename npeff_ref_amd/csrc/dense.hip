@@ -360,8 +360,101 @@ __global__ void __launch_bounds__(256)
   G[(int64_t)b * r + a] = (float)s;
 }
 
+// ---------------------------------------------------------------------------
+// G = X^T X for r <= 32: all of G is one 32x32 MFMA block, and for X^T X the A operand
+// (A[i][k] = X[k][i]) and the B operand (B[k][j] = X[k][j]) of lane (l%32, k = l/32) are the
+// same number, so a wave feeds the MFMA straight from one global load per row pair: no LDS
+// staging, and the kernel runs at the rate the rows stream in.  A wave owns a contiguous run
+// of row pairs; the four waves of a workgroup are summed through LDS into one partial block,
+// and the partials are summed in fp64 by k_gram_small_reduce.
+// ---------------------------------------------------------------------------
+constexpr int GRAM_SMALL_MAX_WGS = 512;
+
+static int64_t gram_small_wgs(int64_t rows) {
+  int64_t s = ceil_div(rows, 1024);
+  if (s > GRAM_SMALL_MAX_WGS) s = GRAM_SMALL_MAX_WGS;
+  if (s < 1) s = 1;
+  return s;
+}
+
+__global__ void __launch_bounds__(256)
+    k_gram_small(const float* __restrict__ X, int64_t rows, int r, float* __restrict__ partials) {
+  __shared__ float red[4 * 1024];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int64_t n_rp = (rows + 1) / 2;
+  const int64_t n_waves = (int64_t)gridDim.x * 4;
+  const int64_t per = (n_rp + n_waves - 1) / n_waves;
+  const int64_t gw = (int64_t)blockIdx.x * 4 + wave;
+  int64_t p0 = gw * per, p1 = p0 + per;
+  if (p0 > n_rp) p0 = n_rp;
+  if (p1 > n_rp) p1 = n_rp;
+  const bool col_ok = l32 < r;
+  const int col = col_ok ? l32 : 0;
+  acc16 acc;
+  for (int v = 0; v < 16; v++) acc[v] = 0.f;
+  int64_t p = p0;
+  // whole groups of GRAM_UNR complete row pairs (an odd row count leaves the last pair of X
+  // without its second row): loads without a bounds check
+  const int64_t p_full = p1 < rows / 2 ? p1 : rows / 2;
+  for (; p + GRAM_UNR <= p_full; p += GRAM_UNR) {
+    float x[GRAM_UNR];
+#pragma unroll
+    for (int u = 0; u < GRAM_UNR; u++) x[u] = X[(2 * (p + u) + half) * r + col];
+#pragma unroll
+    for (int u = 0; u < GRAM_UNR; u++) {
+      const float v = col_ok ? x[u] : 0.f;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(v, v, acc, 0, 0, 0);
+    }
+  }
+  for (; p < p1; p++) {
+    const int64_t row = 2 * p + half;
+    const bool ok = col_ok && row < rows;
+    const float v = ok ? X[(row < rows ? row : rows - 1) * r + col] : 0.f;
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(v, v, acc, 0, 0, 0);
+  }
+  // D layout of the 32x32 block: reg v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+  for (int v = 0; v < 16; v++) red[wave * 1024 + (8 * (v >> 2) + 4 * half + (v & 3)) * 32 + l32] = acc[v];
+  __syncthreads();
+  float* out = partials + (int64_t)blockIdx.x * 1024;
+  for (int e = threadIdx.x; e < 1024; e += 256)
+    out[e] = (red[e] + red[1024 + e]) + (red[2048 + e] + red[3072 + e]);
+}
+
+// One workgroup per row of G: 8 groups of 32 threads each sum every 8th partial (four loads in
+// flight), then the 8 sums are added in fp64 through LDS.
+__global__ void __launch_bounds__(256)
+    k_gram_small_reduce(const float* __restrict__ partials, int64_t n_parts, int r,
+                        float* __restrict__ G) {
+  __shared__ double red[256];
+  const int a = blockIdx.x, b = threadIdx.x & 31, g = threadIdx.x >> 5;
+  const float* p = partials + a * 32 + b;
+  double s = 0.0;
+  int64_t q = g;
+  for (; q + 24 < n_parts; q += 32) {
+    const float x0 = p[q * 1024], x1 = p[(q + 8) * 1024], x2 = p[(q + 16) * 1024],
+                x3 = p[(q + 24) * 1024];
+    s += ((double)x0 + (double)x1) + ((double)x2 + (double)x3);
+  }
+  for (; q < n_parts; q += 8) s += (double)p[q * 1024];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  if (g == 0 && b < r) {
+    for (int k = 1; k < 8; k++) s += red[k * 32 + b];
+    G[a * r + b] = (float)s;
+  }
+}
+
 int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace) {
   DN_CHECK(r >= 1 && r <= 1024, "rank %d outside [1, 1024]", r);
+  if (r <= 32 && rows >= 1) {
+    const int64_t wgs = gram_small_wgs(rows);
+    hipLaunchKernelGGL(k_gram_small, dim3((unsigned)wgs), dim3(256), 0, stream(), X, rows, r,
+                       workspace);
+    hipLaunchKernelGGL(k_gram_small_reduce, dim3((unsigned)r), dim3(256), 0, stream(), workspace, wgs, r, G);
+    DN_LAUNCH_CHECK();
+    return 0;
+  }
   if (gram_uses_tiles(rows, r) && ((uintptr_t)X % 16) == 0)
     return launch_gram_tiles(rows, r, X, G, workspace);
   const int n_pairs = gram_pairs(r);

@@ -71,7 +71,7 @@ def test_spmm_long_rows_and_long_columns():
     A.close()
 
 
-@pytest.mark.parametrize("rows,r", [(1, 16), (31, 16), (1000, 50), (4097, 128), (20000, 256), (9000, 512), (300, 130),
+@pytest.mark.parametrize("rows,r", [(1, 16), (31, 16), (2, 1), (100001, 7), (70000, 32), (333333, 24), (1000, 50), (4097, 128), (20000, 256), (9000, 512), (300, 130),
                                      (1025, 1024), (5000, 384), (1023, 256)])
 def test_gram(rows, r):
     rng = np.random.default_rng(rows + r)
