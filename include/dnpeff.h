@@ -328,6 +328,14 @@ int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr);
 int dnpeff_op_xg_mu(int64_t rows, int r, const float* X, const float* G_rr,
                     const float* num, float eps, float* out, float* D_out);
 
+/* The same update for r = 128 that also returns the Gram matrix of its result:
+ * out = X * num / (X G + eps), Gout = out^T out, in one pass over the rows
+ * (rows >= 64; out may alias num but not X).  This is what dnpeff_nmf_update_H
+ * runs at rank 128; the reference has no counterpart (it calls cublasSgemm for
+ * H^T H separately, device_contexts1.h:303).  For tests and benchmarks. */
+int dnpeff_op_xg_mu_gram(int64_t rows, const float* X, const float* G_rr,
+                         const float* num, float eps, float* out, float* Gout_rr);
+
 /* <x, y> over count floats, fp64 accumulation; result to the host.
  * frobeniusProductToHost (device_contexts1.h:503-537). */
 int dnpeff_op_dot(int64_t count, const float* x, const float* y, double* out_host);

@@ -34,6 +34,7 @@ from .binding import (  # noqa: F401
     op_spmm_t,
     op_gram,
     op_xg_mu,
+    op_xg_mu_gram,
     op_dot,
     op_spsp_dense,
     op_init_uniform,

@@ -101,6 +101,7 @@ SIGNATURES = {
     "dnpeff_op_spmm_t": (C.c_int, [_p, C.c_int, _p, _p]),
     "dnpeff_op_gram": (C.c_int, [_i64, C.c_int, _p, _p]),
     "dnpeff_op_xg_mu": (C.c_int, [_i64, C.c_int, _p, _p, _p, _f32, _p, _p]),
+    "dnpeff_op_xg_mu_gram": (C.c_int, [_i64, _p, _p, _p, _f32, _p, _p]),
     "dnpeff_op_dot": (C.c_int, [_i64, _p, _p, C.POINTER(_f64)]),
     "dnpeff_op_spsp_dense": (C.c_int, [_p, _p, _p]),
     "dnpeff_op_copy": (C.c_int, [_i64, _p, _p]),
@@ -227,6 +228,13 @@ def op_xg_mu(X: DeviceArray, G: DeviceArray, num: DeviceArray, eps: float, out: 
         lib.dnpeff_op_xg_mu(X.shape[0], X.shape[1], X.ptr, G.ptr, num.ptr, eps, out.ptr,
                             None if D_out is None else D_out.ptr)
     )
+
+
+def op_xg_mu_gram(X: DeviceArray, G: DeviceArray, num: DeviceArray, eps: float, out: DeviceArray,
+                  Gout: DeviceArray):
+    """Rank 128: out = X * num / (X G + eps) and Gout = out^T out in one pass."""
+    assert X.shape[1] == 128
+    _check(lib.dnpeff_op_xg_mu_gram(X.shape[0], X.ptr, G.ptr, num.ptr, eps, out.ptr, Gout.ptr))
 
 
 def op_dot(x: DeviceArray, y: DeviceArray) -> float:

@@ -1188,7 +1188,10 @@ __global__ void __launch_bounds__(256)
     return (3 * w + k) * 1024 + (4 * (ii >> 3) + (ii & 3)) * 64 + jj + 32 * ((ii >> 2) & 1);
   };
   double s = 0.0;
-  if (ca <= cbk) {
+  // of a diagonal block only the upper triangle: the split-operand kernel's (i, j) and (j, i)
+  // sums differ in their last bits, and Gout must be exactly symmetric
+  const bool mine = ca < cbk || (ca == cbk && i <= j);
+  if (mine) {
     int src0, src1 = -1;
     switch (cbk - ca) {
       case 0: src0 = at(ca, 0, i, j); break;
@@ -1205,7 +1208,7 @@ __global__ void __launch_bounds__(256)
   }
   red[q][threadIdx.x & 31] = s;
   __syncthreads();
-  if (q == 0 && ca <= cbk) {
+  if (q == 0 && mine) {
     double t = 0.0;
     for (int u = 0; u < 8; u++) t += red[u][threadIdx.x];
     Gout[a * 128 + b] = (float)t;
@@ -1213,13 +1216,296 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---------------------------------------------------------------------------
+// The fused update on the bf16 matrix cores, at fp32 accuracy.
+//
+// Every fp32 number is the exact sum of three bf16 numbers, x = h + m + l (each the round-to-
+// nearest bf16 of what the ones before leave; 3 x 8 significant bits cover the 24 of fp32).  A
+// product of two such numbers is then the sum of nine bf16 products, each exact in fp32; the
+// six largest -- hh, hm, mh, hl, lh, mm -- carry everything down to 2^-24 of the result, which
+// is the rounding error of an fp32 multiply.  v_mfma_f32_32x32x16_bf16 contracts 16 components
+// in half the time v_mfma_f32_32x32x2f32 takes for 2, so six of them per 16 components are 2.7
+// times faster than the fp32 matrix cores, with fp32 accumulation either way, and the kernel
+// moves from the matrix-core bound to the HBM bound.
+//
+// Tiles of 32 rows.  X is split once per element on its way into LDS (three bf16 planes
+// [row][k], rows padded to 272 bytes; the next tile is fetched into registers after the MFMAs
+// of the update and stored after those of the Gram part, when no wave reads the planes any
+// more), G is split once per workgroup into registers (lane (j, half) holds the 8
+// components 16 st + 8 half .. + 7 of column j for each of the 8 steps: 32 registers a part).
+// An A operand is one 16-byte LDS read; an fp32 copy of the tile beside the
+// planes gives the epilogue its X factor.  The hardware contracts slot s of lane half `half` of A
+// with the same slot of B, so only the agreement of the two sides matters, not the order of
+// the 16 components inside an instruction.
+//
+// Gram part: the result tile is split again; a lane's registers hold, per column, rows
+// 8 q + 4 half + t -- taken as contraction slots (MFMA u = 0, 1: q = 2u, 2u + 1; t = 0..3) they
+// are the A operand of out^T out directly, and the B operand of the diagonal block.  For the
+// other blocks the parts go to LDS transposed ([column][row], 72 bytes a column), where the
+// four rows of a (q, half) group are 8 contiguous bytes: a B operand is two 8-byte reads.
+// Block ownership, the flush of the accumulators and the partial sums are those of
+// k_xg_mu_gram, with 32-row tiles.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// The two bf16 numbers of a packed pair as floats: a shift and a mask.
+__device__ inline f32x2 widen(const bf16x2& p) {
+  const unsigned u = __builtin_bit_cast(unsigned, p);
+  return f32x2{__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u)};
+}
+// One packed conversion per pair and part; the differences are exact.
+__device__ inline void split3(const f32x2& x, bf16x2& h, bf16x2& m, bf16x2& l) {
+  h = __builtin_convertvector(x, bf16x2);
+  const f32x2 r1 = x - widen(h);
+  m = __builtin_convertvector(r1, bf16x2);
+  const f32x2 r2 = r1 - widen(m);
+  l = __builtin_convertvector(r2, bf16x2);
+}
+__device__ inline void split3(const f32x4& x, bf16x4& h, bf16x4& m, bf16x4& l) {
+  bf16x2 h0, m0, l0, h1, m1, l1;
+  split3(f32x2{x[0], x[1]}, h0, m0, l0);
+  split3(f32x2{x[2], x[3]}, h1, m1, l1);
+  h = __builtin_shufflevector(h0, h1, 0, 1, 2, 3);
+  m = __builtin_shufflevector(m0, m1, 0, 1, 2, 3);
+  l = __builtin_shufflevector(l0, l1, 0, 1, 2, 3);
+}
+__device__ inline bf16x8 cat8(const bf16x4& a, const bf16x4& b) {
+  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+__device__ inline float bf16_bits_to_float(unsigned short u) {
+  return __uint_as_float((unsigned)u << 16);
+}
+
+constexpr int XB_ROWS = 32;
+constexpr int XB_LDX = 272;                  // bytes per row of an X plane
+constexpr int XB_PLANE = XB_ROWS * XB_LDX;
+constexpr int XB_SLOT = 3 * XB_PLANE;
+constexpr int XB_LDO = 72;                   // bytes per column of an out^T plane
+constexpr int XB_OPLANE = 128 * XB_LDO;
+constexpr int XB_LDR = 132;                  // floats per row of the fp32 copy of the X tile
+constexpr int XB_RAW = XB_ROWS * XB_LDR * 4;
+constexpr int XB_LDS = XB_SLOT + 3 * XB_OPLANE + XB_RAW;
+constexpr int XB_FLUSH = 1024;               // tiles between flushes: 32,768 rows
+
+#define DN_MFMA_B16(A, B, C) __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, C, 0, 0, 0)
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_xg_mu_gram_b16(const float* __restrict__ X, const float* __restrict__ G, const float* num,
+                     float eps, int64_t n_tiles, int n_flush, float* out, float* __restrict__ gpart) {
+  constexpr int r = 128;
+  extern __shared__ __align__(16) unsigned char xb[];
+  unsigned char* const oplanes = xb + XB_SLOT;
+  float* const xraw = reinterpret_cast<float*>(xb + XB_SLOT + 3 * XB_OPLANE);
+  const int cb = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int col = 32 * cb + l32;
+
+  bf16x8 gh[8], gm[8], gl[8];
+#pragma unroll
+  for (int st = 0; st < 8; st++) {
+    f32x4 g0, g1;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      g0[s] = G[(16 * st + 8 * half + s) * r + col];
+      g1[s] = G[(16 * st + 8 * half + 4 + s) * r + col];
+    }
+    bf16x4 h0, m0, l0, h1, m1, l1;
+    split3(g0, h0, m0, l0);
+    split3(g1, h1, m1, l1);
+    gh[st] = cat8(h0, h1);
+    gm[st] = cat8(m0, m1);
+    gl[st] = cat8(l0, l1);
+  }
+
+  // a thread fetches 16 bytes of each of 4 rows (8 rows apart): whole rows per wave instruction
+  const int lc = threadIdx.x & 31, lr = threadIdx.x >> 5;
+  f32x4 R[4];
+  auto fetch = [&](int64_t tile) {
+    // past the last tile the loads are redirected to it (and what they bring is never used)
+    const float* src = X + ((tile < n_tiles ? tile : n_tiles - 1) * XB_ROWS + lr) * (int64_t)r + 4 * lc;
+#pragma unroll
+    for (int q = 0; q < 4; q++) R[q] = *reinterpret_cast<const f32x4*>(src + q * 8 * r);
+  };
+  auto commit = [&](unsigned char* slot) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      bf16x4 h, m, l;
+      split3(R[q], h, m, l);
+      unsigned char* dst = slot + (lr + 8 * q) * XB_LDX + 8 * lc;
+      *reinterpret_cast<bf16x4*>(dst) = h;
+      *reinterpret_cast<bf16x4*>(dst + XB_PLANE) = m;
+      *reinterpret_cast<bf16x4*>(dst + 2 * XB_PLANE) = l;
+      *reinterpret_cast<f32x4*>(xraw + (lr + 8 * q) * XB_LDR + 4 * lc) = R[q];
+    }
+  };
+
+  acc16 ga[3];
+  auto ga_clear = [&]() {
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) ga[k][v] = 0.0f;
+  };
+  auto ga_flush = [&](int chunk) {
+    float* dst = gpart + (((int64_t)blockIdx.x * n_flush + chunk) * XGG_BLOCKS + 3 * cb) * 1024 + lane;
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) dst[k * 1024 + v * 64] = ga[k][v];
+  };
+  ga_clear();
+
+  int64_t tile = blockIdx.x;
+  fetch(tile);
+  commit(xb);
+  const unsigned off0 = (unsigned)(4 * half * r + col);
+  // numerators of a tile in the accumulator layout; past the last tile the loads are
+  // redirected to it (and their values never used)
+  float pn[16], pnn[16];
+  auto numerators = [&](int64_t t, float (&dst)[16]) {
+    const float* tnum = num + (t < n_tiles ? t : n_tiles - 1) * XB_ROWS * (int64_t)r;
+#pragma unroll
+    for (int v = 0; v < 16; v++) dst[v] = (tnum + (8 * (v >> 2) + (v & 3)) * r)[off0];
+  };
+  numerators(tile, pn);
+  __syncthreads();
+
+  const int cb1 = (cb + 1) & 3, cb2 = (cb + 2) & 3;
+  int it = 0;
+  for (; tile < n_tiles; it++, tile += gridDim.x) {
+    const unsigned char* slot = xb;
+    float* tout = out + tile * XB_ROWS * (int64_t)r;
+    // the next tile and its numerators travel during this iteration
+    fetch(tile + gridDim.x);
+
+    acc16 a0;
+#pragma unroll
+    for (int v = 0; v < 16; v++) a0[v] = 0.0f;
+    const unsigned char* arow = slot + l32 * XB_LDX + 16 * half;
+#pragma unroll
+    for (int st = 0; st < 8; st++) {
+      const bf16x8 xh = *reinterpret_cast<const bf16x8*>(arow + 32 * st);
+      const bf16x8 xm = *reinterpret_cast<const bf16x8*>(arow + 32 * st + XB_PLANE);
+      const bf16x8 xl = *reinterpret_cast<const bf16x8*>(arow + 32 * st + 2 * XB_PLANE);
+      a0 = DN_MFMA_B16(xh, gh[st], a0);
+      a0 = DN_MFMA_B16(xh, gm[st], a0);
+      a0 = DN_MFMA_B16(xm, gh[st], a0);
+      a0 = DN_MFMA_B16(xh, gl[st], a0);
+      a0 = DN_MFMA_B16(xl, gh[st], a0);
+      a0 = DN_MFMA_B16(xm, gm[st], a0);
+    }
+    numerators(tile + gridDim.x, pnn);
+
+    // epilogue: the result replaces the numerators
+    {
+      float x[16];
+#pragma unroll
+      for (int v = 0; v < 16; v++) x[v] = xraw[(8 * (v >> 2) + 4 * half + (v & 3)) * XB_LDR + col];
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        // quotient from the reciprocal (1 ulp) and one correction step
+        const float den = a0[v] + eps, rc = __builtin_amdgcn_rcpf(den);
+        const float q0 = pn[v] * rc;
+        const float q = __builtin_fmaf(__builtin_fmaf(-den, q0, pn[v]), rc, q0);
+        const float o = x[v] * q;
+        pn[v] = o;
+        (tout + (8 * (v >> 2) + (v & 3)) * r)[off0] = o;
+      }
+    }
+    // parts of the result: registers for the A side, LDS (transposed) for the other waves.
+    // The planes were last read before the barrier that ended the previous iteration.
+    bf16x4 oh[4], om[4], ol[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const f32x4 o = {pn[4 * q], pn[4 * q + 1], pn[4 * q + 2], pn[4 * q + 3]};
+      split3(o, oh[q], om[q], ol[q]);
+      unsigned char* dst = oplanes + col * XB_LDO + 2 * (8 * q + 4 * half);
+      *reinterpret_cast<bf16x4*>(dst) = oh[q];
+      *reinterpret_cast<bf16x4*>(dst + XB_OPLANE) = om[q];
+      *reinterpret_cast<bf16x4*>(dst + 2 * XB_OPLANE) = ol[q];
+    }
+    __syncthreads();
+
+    // Gram blocks of the new tile; the block pairs two apart, (0, 2) and (1, 3), are taken by
+    // waves 0 and 1 on even iterations and, transposed, by waves 2 and 3 on odd ones
+    const bool third = (cb < 2) == ((it & 1) == 0);
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const bf16x8 ah = cat8(oh[2 * u], oh[2 * u + 1]);
+      const bf16x8 am = cat8(om[2 * u], om[2 * u + 1]);
+      const bf16x8 al = cat8(ol[2 * u], ol[2 * u + 1]);
+      auto side = [&](int cbb, int part) {
+        const unsigned char* p =
+            oplanes + part * XB_OPLANE + (32 * cbb + l32) * XB_LDO + 2 * (16 * u + 4 * half);
+        return cat8(*reinterpret_cast<const bf16x4*>(p), *reinterpret_cast<const bf16x4*>(p + 16));
+      };
+      const bf16x8 bh = side(cb1, 0), bm = side(cb1, 1), bl = side(cb1, 2);
+      ga[0] = DN_MFMA_B16(ah, ah, ga[0]);
+      ga[1] = DN_MFMA_B16(ah, bh, ga[1]);
+      ga[0] = DN_MFMA_B16(ah, am, ga[0]);
+      ga[1] = DN_MFMA_B16(ah, bm, ga[1]);
+      ga[0] = DN_MFMA_B16(am, ah, ga[0]);
+      ga[1] = DN_MFMA_B16(am, bh, ga[1]);
+      ga[0] = DN_MFMA_B16(ah, al, ga[0]);
+      ga[1] = DN_MFMA_B16(ah, bl, ga[1]);
+      ga[0] = DN_MFMA_B16(al, ah, ga[0]);
+      ga[1] = DN_MFMA_B16(al, bh, ga[1]);
+      ga[0] = DN_MFMA_B16(am, am, ga[0]);
+      ga[1] = DN_MFMA_B16(am, bm, ga[1]);
+      if (third) {
+        const bf16x8 ch = side(cb2, 0), cm = side(cb2, 1), cl = side(cb2, 2);
+        ga[2] = DN_MFMA_B16(ah, ch, ga[2]);
+        ga[2] = DN_MFMA_B16(ah, cm, ga[2]);
+        ga[2] = DN_MFMA_B16(am, ch, ga[2]);
+        ga[2] = DN_MFMA_B16(ah, cl, ga[2]);
+        ga[2] = DN_MFMA_B16(al, ch, ga[2]);
+        ga[2] = DN_MFMA_B16(am, cm, ga[2]);
+      }
+    }
+    if ((it + 1) % XB_FLUSH == 0) {
+      ga_flush(it / XB_FLUSH);
+      ga_clear();
+    }
+
+    // every wave has left the X planes behind at the barrier above: they take the next tile
+    commit(xb);
+#pragma unroll
+    for (int v = 0; v < 16; v++) pn[v] = pnn[v];
+    __syncthreads();
+  }
+  // the chunk in progress, then zeros for the chunks this workgroup never reached
+  int chunk = it / XB_FLUSH;
+  if (it % XB_FLUSH != 0 || it == 0) ga_flush(chunk++);
+  ga_clear();
+  for (; chunk < n_flush; chunk++) ga_flush(chunk);
+}
+
 // Workspace of the fused update in floats, for `rows` rows.
-int64_t xg_mu_gram_workspace_floats(int64_t rows) {
-  const int64_t tiles = rows / XgReg<4>::ROWS;
+static int64_t xgg_parts(int64_t rows, int tile_rows, int flush, int64_t* wgs_out, int64_t* n_flush_out) {
+  const int64_t tiles = rows / tile_rows;
   int64_t wgs = (int64_t)n_cus() * 2;
   if (wgs > tiles) wgs = tiles > 0 ? tiles : 1;
-  const int64_t n_flush = ceil_div(ceil_div(tiles > 0 ? tiles : 1, wgs), XGG_FLUSH);
-  return wgs * n_flush * XGG_BLOCKS * 1024;
+  const int64_t n_flush = ceil_div(ceil_div(tiles > 0 ? tiles : 1, wgs), flush);
+  if (wgs_out) *wgs_out = wgs;
+  if (n_flush_out) *n_flush_out = n_flush;
+  return wgs * n_flush;
+}
+
+// The bf16-split kernel is the default; DNPEFF_SPLIT_BF16=0 selects the fp32 matrix-core one.
+static bool use_split_bf16() {
+  const char* e = getenv("DNPEFF_SPLIT_BF16");
+  return e ? atoi(e) != 0 : true;
+}
+
+int64_t xg_mu_gram_workspace_floats(int64_t rows) {
+  const int64_t a = xgg_parts(rows, XgReg<4>::ROWS, XGG_FLUSH, nullptr, nullptr);
+  const int64_t b = xgg_parts(rows, XB_ROWS, XB_FLUSH, nullptr, nullptr);
+  return (a > b ? a : b) * XGG_BLOCKS * 1024;
 }
 
 // out = X * num / (X G + eps) and Gout = out^T out for r = 128; rows >= 64.  The rows past the
@@ -1234,24 +1520,30 @@ int launch_xg_mu_gram(int64_t rows, const float* X, const float* G, const float*
                       float* out, float* Gout, float* gpart, float* G_tmp, float* gram_ws) {
   using C = XgReg<4>;
   constexpr int r = 128;
-  const size_t lds = sizeof(float) * 2 * C::SLOT;
-  static bool attr_set = false;
-  if (!attr_set) {
-    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_gram, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)lds));
-    attr_set = true;
+  const bool split = use_split_bf16();
+  const int tile_rows = split ? XB_ROWS : C::ROWS;
+  const size_t lds = split ? (size_t)XB_LDS : sizeof(float) * 2 * C::SLOT;
+  static bool attr_set[2] = {false, false};
+  if (!attr_set[split]) {
+    DN_HIP(hipFuncSetAttribute(split ? (const void*)k_xg_mu_gram_b16 : (const void*)k_xg_mu_gram,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set[split] = true;
   }
-  const int64_t tiles = rows / C::ROWS;
+  const int64_t tiles = rows / tile_rows;
   DN_CHECK(tiles >= 1, "fused update needs at least one whole tile");
-  int64_t wgs = (int64_t)n_cus() * 2;
-  if (wgs > tiles) wgs = tiles;
-  const int64_t n_flush = ceil_div(ceil_div(tiles, wgs), XGG_FLUSH);
-  hipLaunchKernelGGL(k_xg_mu_gram, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps, tiles,
-                     (int)n_flush, out, gpart);
+  DN_CHECK(((uintptr_t)X % 16) == 0, "fused update: X must be 16-byte aligned");
+  int64_t wgs, n_flush;
+  xgg_parts(rows, tile_rows, split ? XB_FLUSH : XGG_FLUSH, &wgs, &n_flush);
+  if (split)
+    hipLaunchKernelGGL(k_xg_mu_gram_b16, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps,
+                       tiles, (int)n_flush, out, gpart);
+  else
+    hipLaunchKernelGGL(k_xg_mu_gram, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps, tiles,
+                       (int)n_flush, out, gpart);
   hipLaunchKernelGGL(k_xg_gram_reduce, dim3(128 * 128 / 32), dim3(256), 0, stream(), gpart,
                      wgs * n_flush, Gout);
   DN_LAUNCH_CHECK();
-  const int64_t head = tiles * C::ROWS;
+  const int64_t head = tiles * tile_rows;
   if (head < rows) {
     const int64_t off = head * r;
     DN_TRY(launch_xg_mu_nb<4>(rows - head, r, X + off, G, num + off, eps, out + off, nullptr));
@@ -1260,6 +1552,25 @@ int launch_xg_mu_gram(int64_t rows, const float* X, const float* G, const float*
     DN_LAUNCH_CHECK();
   }
   return 0;
+}
+
+// Kernel-level entry point of the fused update (rank 128): allocates its workspaces per call.
+DN_API int dnpeff_op_xg_mu_gram(int64_t rows, const float* X, const float* G_rr, const float* num,
+                                float eps, float* out, float* Gout_rr) {
+  clear_error();
+  DN_CHECK(rows >= 64, "fused update needs at least 64 rows");
+  float *gpart = nullptr, *G_tmp = nullptr, *gram_ws = nullptr;
+  int s = dmalloc(&gpart, xg_mu_gram_workspace_floats(rows)) || dmalloc(&G_tmp, 128 * 128) ||
+          dmalloc(&gram_ws, gram_workspace_floats(64, 128));
+  if (!s) s = launch_xg_mu_gram(rows, X, G_rr, num, eps, out, Gout_rr, gpart, G_tmp, gram_ws);
+  if (!s && hipStreamSynchronize(stream()) != hipSuccess) {
+    set_error("fused update: kernel failed");
+    s = 1;
+  }
+  dfree(gpart);
+  dfree(G_tmp);
+  dfree(gram_ws);
+  return s;
 }
 
 int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const float* num, float eps,

@@ -24,7 +24,7 @@ import npeff_ref_amd as d  # noqa: E402
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--op", required=True, choices=["mu", "gram", "xg_mu", "copy", "spmm_n", "spmm_t", "topk"])
+    ap.add_argument("--op", required=True, choices=["mu", "gram", "xg_mu", "xg_mu_gram", "copy", "spmm_n", "spmm_t", "topk"])
     ap.add_argument("--rows", type=int, default=4_000_000)
     ap.add_argument("--rank", type=int, default=128)
     ap.add_argument("--iters", type=int, default=5)
@@ -73,6 +73,11 @@ def main():
             G, num, out = uniform(r, r, 4), uniform(rows, r, 5), d.DeviceArray((rows, r))
             fn = lambda: d.op_xg_mu(X, G, num, 1e-12, out)
             work = 2 * rows * r * r
+        elif a.op == "xg_mu_gram":
+            # the H update of the factorisation at rank 128: in place on the numerator
+            G, num, Gout = uniform(r, r, 4), uniform(rows, r, 5), d.DeviceArray((r, r))
+            fn = lambda: d.op_xg_mu_gram(X, G, num, 1e-12, num, Gout)
+            work = 12 * rows * r
         elif a.op == "mu":
             num, den = uniform(rows, r, 5), uniform(rows, r, 6)
             fn = lambda: d.op_mu(X, num, den, 1e-12)

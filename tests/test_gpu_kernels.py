@@ -105,6 +105,38 @@ def test_xg_mu(rows, r):
     assert np.array_equal(dnum.numpy(), out1)
 
 
+@pytest.mark.parametrize("split", ["1", "0"])
+@pytest.mark.parametrize("rows", [64, 95, 4100, 70001, 300033])
+def test_xg_mu_gram_fused(rows, split, monkeypatch):
+    """Rank 128, update and Gram matrix of the result in one pass: on the bf16 matrix cores with
+    every operand split in three (default) and on the fp32 ones.  Both must meet the fp32 bar;
+    the operands span 12 decades and hold zeros, so the split's low parts matter."""
+    monkeypatch.setenv("DNPEFF_SPLIT_BF16", split)
+    r = 128
+    rng = np.random.default_rng(rows)
+    X = (rng.random((rows, r)) * 10.0 ** rng.uniform(-6, 0, (rows, r))).astype(np.float32)
+    X[rng.random((rows, r)) < 0.05] = 0.0
+    G = (rng.random((r, r)) * 10.0 ** rng.uniform(-3, 3, (r, r))).astype(np.float32)
+    num = (rng.random((rows, r)) * 10.0 ** rng.uniform(-3, 3, (rows, r))).astype(np.float32)
+    eps = np.float32(1e-12)
+    dX, dG, dnum = d.DeviceArray.from_numpy(X), d.DeviceArray.from_numpy(G), d.DeviceArray.from_numpy(num)
+    dout, dGo = d.DeviceArray((rows, r)), d.DeviceArray((r, r))
+    d.op_xg_mu_gram(dX, dG, dnum, eps, dout, dGo)
+    want, _ = orc.xg_mu_f64(X, G, num, eps)
+    out = dout.numpy()
+    # element-wise: every entry to a few fp32 ulps, not only the norm
+    ok = np.abs(out - want) <= 2e-6 * np.abs(want) + 1e-30
+    assert ok.all(), float(np.max(np.abs(out - want) / (np.abs(want) + 1e-30)))
+    Go = dGo.numpy()
+    wantG = orc.gram_f64(out)
+    assert _rel(Go, wantG) < 2e-6
+    assert np.array_equal(Go, Go.T)
+    # in place on the numerator buffer gives the same bits
+    d.op_xg_mu_gram(dX, dG, dnum, eps, dnum, dGo)
+    assert np.array_equal(dnum.numpy(), out)
+    assert np.array_equal(dGo.numpy(), Go)
+
+
 def test_dot_fp64_accumulation():
     rng = np.random.default_rng(1)
     n = 3_000_001
