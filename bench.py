@@ -51,9 +51,12 @@ def log(msg):
     print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
 
 
-def algorithmic(cls, n, m, z, r, fused_gram=False):
+def algorithmic(cls, n, m, z, r, fused_gram=False, split_bf16=False):
     """Compulsory traffic / flops of one launch: every operand touched once.  With fused_gram the
-    H update also produces H^T H (no separate gram_H launch): its class carries both products."""
+    H update also produces H^T H (no separate gram_H launch): its class carries both products.
+    With split_bf16 those products run on the bf16 matrix cores (every fp32 operand as the sum of
+    three bf16 numbers, six partial products, fp32 accumulation), whose peak is 16 times the fp32
+    cores': the launch is then bounded by its three passes over m x r floats, not by arithmetic."""
     P = 4 if z < 2**31 else 8
     if cls == "spmm_n":
         return "hbm", 8 * z + P * (n + 1) + 4 * r * m + 4 * n * r
@@ -67,6 +70,8 @@ def algorithmic(cls, n, m, z, r, fused_gram=False):
     if cls == "gram_W":
         return ("mfma", n * r * (r + 1)) if r >= 64 else ("hbm", 4 * n * r + 4 * r * r)
     if cls == "xg_mu_H":
+        if fused_gram and split_bf16:
+            return "hbm", 12 * m * r + 8 * r * r
         if fused_gram:
             return "mfma", 2 * m * r * r + m * r * (r + 1)
         return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 12 * m * r + 4 * r * r)
@@ -175,10 +180,11 @@ def main():
 
     kernels = {}
     fused_gram = tim.get("gram_H", (0.0, 0))[1] == 0
+    split_bf16 = fused_gram and os.environ.get("DNPEFF_SPLIT_BF16", "1") != "0"
     for cls, (ms_sum, cnt) in tim.items():
         if cnt == 0:
             continue
-        bound, work = algorithmic(cls, n, m, z, r, fused_gram)
+        bound, work = algorithmic(cls, n, m, z, r, fused_gram, split_bf16)
         avg_s = ms_sum / cnt * 1e-3
         peak = HBM_PEAK if bound == "hbm" else MFMA_FP32_PEAK
         kernels[cls] = dict(
@@ -219,6 +225,8 @@ def main():
         "cpu_baseline": cpu_baseline,
         "kernels": kernels,
         "fused_gram_in_H_update": fused_gram,
+        "h_update_products": ("bf16 MFMA on fp32 operands split in three (6 partial products, fp32 "
+                              "accumulation, fp32 accuracy)" if split_bf16 else "fp32 MFMA"),
         "spmm_hbm_frac": {k: kernels[k]["frac"] for k in ("spmm_n", "spmm_t") if k in kernels},
         "loss_after": loss,
     }

@@ -638,6 +638,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 // reads and stores the compiler batches; code for partial tiles would cost registers that the
 // main path needs.
 // ---------------------------------------------------------------------------
+// Consecutive tiles a workgroup takes at a time: a power of two, 16 where that leaves every
+// workgroup several runs, less for short inputs.
+static int xg_run(int64_t tiles, int64_t wgs_max) {
+  int run = 16;
+  while (run > 1 && tiles / run < 4 * wgs_max) run /= 2;
+  return run;
+}
+
 template <int CB>
 struct XgReg {
   static constexpr int WPC = 4 / CB;         // waves per column block
@@ -655,7 +663,7 @@ struct XgReg {
 template <int CB, bool WITH_D>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_xg_mu_reg(const float* __restrict__ X, const float* __restrict__ G, const float* num,
-                float eps, int64_t n_tiles, float* out, float* __restrict__ D_out) {
+                float eps, int64_t n_tiles, int run, float* out, float* __restrict__ D_out) {
   using C = XgReg<CB>;
   constexpr int r = C::R;
   extern __shared__ __align__(16) float xl[];  // 2 slots of ROWS x LD
@@ -685,10 +693,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       *reinterpret_cast<float4*>(slot + (lr + q * C::RSTEP) * C::LD + 4 * lc) = R[q];
   };
 
-  int64_t tile = blockIdx.x;
+  // A workgroup takes runs of `run` (a power of two) consecutive tiles, the runs dealt
+  // round-robin (single tiles dealt round-robin put a workgroup's tiles a fixed power-of-two
+  // stride apart, which costs about 15 % of the streaming rate).
+  auto after = [&](int64_t t) {
+    return ((t + 1) & (run - 1)) != 0 ? t + 1 : t + 1 + ((int64_t)gridDim.x - 1) * run;
+  };
+  int64_t tile = (int64_t)blockIdx.x * run;
   fetch(tile);
   commit(xl);
-  fetch(tile + gridDim.x);
+  fetch(after(tile));
   __syncthreads();
 
   // element (b, v) of the accumulators sits 32 b + 8 (v / 4) + v % 4 rows below the lane's
@@ -696,7 +710,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int lrow0 = 32 * C::RB * rg + 4 * half;
   const unsigned off0 = (unsigned)(lrow0 * r + col);
 
-  for (int it = 0; tile < n_tiles; it++, tile += gridDim.x) {
+  for (int it = 0; tile < n_tiles; it++, tile = after(tile)) {
     const float* slot = xl + (it & 1) * C::SLOT;
     const int64_t t0 = tile * C::ROWS * (int64_t)r;
     const float* tnum = num + t0;
@@ -750,7 +764,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // the other slot was last read before the previous barrier: it takes the next tile, whose
     // loads were issued one tile ago; the registers then take the tile after it
     commit(xl + ((it + 1) & 1) * C::SLOT);
-    fetch(tile + 2 * (int64_t)gridDim.x);
+    fetch(after(after(tile)));
     __syncthreads();
   }
 }
@@ -772,14 +786,15 @@ static int launch_xg_mu_reg(int64_t rows, const float* X, const float* G, const 
   const int64_t tiles = rows / C::ROWS;
   if (tiles == 0) return 0;
   int64_t wgs = (int64_t)n_cus() * 2;
-  if (wgs > tiles) wgs = tiles;
+  const int run = xg_run(tiles, wgs);
+  if (wgs > ceil_div(tiles, run)) wgs = ceil_div(tiles, run);
   const dim3 grid((unsigned)wgs), block(256);
   if (D_out)
     hipLaunchKernelGGL((k_xg_mu_reg<CB, true>), grid, block, lds, stream(), X, G, num, eps, tiles,
-                       out, D_out);
+                       run, out, D_out);
   else
     hipLaunchKernelGGL((k_xg_mu_reg<CB, false>), grid, block, lds, stream(), X, G, num, eps, tiles,
-                       out, D_out);
+                       run, out, D_out);
   DN_LAUNCH_CHECK();
   return 0;
 }
@@ -1296,7 +1311,8 @@ constexpr int XB_FLUSH = 1024;               // tiles between flushes: 32,768 ro
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_xg_mu_gram_b16(const float* __restrict__ X, const float* __restrict__ G, const float* num,
-                     float eps, int64_t n_tiles, int n_flush, float* out, float* __restrict__ gpart) {
+                     float eps, int64_t n_tiles, int run, int n_flush, float* out,
+                     float* __restrict__ gpart) {
   constexpr int r = 128;
   extern __shared__ __align__(16) unsigned char xb[];
   unsigned char* const oplanes = xb + XB_SLOT;
@@ -1360,7 +1376,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   };
   ga_clear();
 
-  int64_t tile = blockIdx.x;
+  // A workgroup takes runs of `run` (a power of two) consecutive tiles, the runs dealt
+  // round-robin: with single tiles dealt round-robin, the tiles of a workgroup lie a fixed
+  // power-of-two stride apart, and the three streams then reach 4.4 TB/s where runs reach 5.2.
+  auto after = [&](int64_t t) {
+    return ((t + 1) & (run - 1)) != 0 ? t + 1 : t + 1 + ((int64_t)gridDim.x - 1) * run;
+  };
+  int64_t tile = (int64_t)blockIdx.x * run;
   fetch(tile);
   commit(xb);
   const unsigned off0 = (unsigned)(4 * half * r + col);
@@ -1377,11 +1399,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   const int cb1 = (cb + 1) & 3, cb2 = (cb + 2) & 3;
   int it = 0;
-  for (; tile < n_tiles; it++, tile += gridDim.x) {
+  for (; tile < n_tiles; it++, tile = after(tile)) {
     const unsigned char* slot = xb;
     float* tout = out + tile * XB_ROWS * (int64_t)r;
     // the next tile and its numerators travel during this iteration
-    fetch(tile + gridDim.x);
+    fetch(after(tile));
 
     acc16 a0;
 #pragma unroll
@@ -1399,7 +1421,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       a0 = DN_MFMA_B16(xl, gh[st], a0);
       a0 = DN_MFMA_B16(xm, gm[st], a0);
     }
-    numerators(tile + gridDim.x, pnn);
+    numerators(after(tile), pnn);
 
     // epilogue: the result replaces the numerators
     {
@@ -1485,12 +1507,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   for (; chunk < n_flush; chunk++) ga_flush(chunk);
 }
 
-// Workspace of the fused update in floats, for `rows` rows.
-static int64_t xgg_parts(int64_t rows, int tile_rows, int flush, int64_t* wgs_out, int64_t* n_flush_out) {
+// Number of partial Gram matrices of the fused update (workgroups x flushes) for `rows` rows;
+// runs_of_tiles: a workgroup takes several consecutive tiles at a time (xg_run) instead of one.
+static int64_t xgg_parts(int64_t rows, int tile_rows, int flush, bool runs_of_tiles, int64_t* wgs_out,
+                         int64_t* n_flush_out, int* run_out = nullptr) {
   const int64_t tiles = rows / tile_rows;
   int64_t wgs = (int64_t)n_cus() * 2;
-  if (wgs > tiles) wgs = tiles > 0 ? tiles : 1;
-  const int64_t n_flush = ceil_div(ceil_div(tiles > 0 ? tiles : 1, wgs), flush);
+  const int run = runs_of_tiles ? xg_run(tiles, wgs) : 1;
+  if (run_out) *run_out = run;
+  const int64_t runs = ceil_div(tiles > 0 ? tiles : 1, run);
+  if (wgs > runs) wgs = runs;
+  const int64_t n_flush = ceil_div(ceil_div(runs, wgs) * run, flush);
   if (wgs_out) *wgs_out = wgs;
   if (n_flush_out) *n_flush_out = n_flush;
   return wgs * n_flush;
@@ -1502,9 +1529,10 @@ static bool use_split_bf16() {
   return e ? atoi(e) != 0 : true;
 }
 
+// Workspace of the fused update in floats, for `rows` rows.
 int64_t xg_mu_gram_workspace_floats(int64_t rows) {
-  const int64_t a = xgg_parts(rows, XgReg<4>::ROWS, XGG_FLUSH, nullptr, nullptr);
-  const int64_t b = xgg_parts(rows, XB_ROWS, XB_FLUSH, nullptr, nullptr);
+  const int64_t a = xgg_parts(rows, XgReg<4>::ROWS, XGG_FLUSH, false, nullptr, nullptr);
+  const int64_t b = xgg_parts(rows, XB_ROWS, XB_FLUSH, true, nullptr, nullptr);
   return (a > b ? a : b) * XGG_BLOCKS * 1024;
 }
 
@@ -1533,10 +1561,11 @@ int launch_xg_mu_gram(int64_t rows, const float* X, const float* G, const float*
   DN_CHECK(tiles >= 1, "fused update needs at least one whole tile");
   DN_CHECK(((uintptr_t)X % 16) == 0, "fused update: X must be 16-byte aligned");
   int64_t wgs, n_flush;
-  xgg_parts(rows, tile_rows, split ? XB_FLUSH : XGG_FLUSH, &wgs, &n_flush);
+  int run;
+  xgg_parts(rows, tile_rows, split ? XB_FLUSH : XGG_FLUSH, split, &wgs, &n_flush, &run);
   if (split)
     hipLaunchKernelGGL(k_xg_mu_gram_b16, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps,
-                       tiles, (int)n_flush, out, gpart);
+                       tiles, run, (int)n_flush, out, gpart);
   else
     hipLaunchKernelGGL(k_xg_mu_gram, dim3((unsigned)wgs), dim3(256), lds, stream(), X, G, num, eps, tiles,
                        (int)n_flush, out, gpart);
