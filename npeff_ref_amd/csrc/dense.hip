@@ -3,6 +3,7 @@
 // multiplicative update fused into the X G epilogue, dot products with fp64
 // accumulation, seeded initialisation and the [m, r] <-> [r, m] transposition.
 #include "dnpeff_internal.hpp"
+#include "split_bf16.hpp"
 #include "synth_rng.h"
 
 #include <type_traits>
@@ -1261,41 +1262,6 @@ __global__ void __launch_bounds__(256)
 // Block ownership, the flush of the accumulators and the partial sums are those of
 // k_xg_mu_gram, with 32-row tiles.
 // ---------------------------------------------------------------------------
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-// The two bf16 numbers of a packed pair as floats: a shift and a mask.
-__device__ inline f32x2 widen(const bf16x2& p) {
-  const unsigned u = __builtin_bit_cast(unsigned, p);
-  return f32x2{__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u)};
-}
-// One packed conversion per pair and part; the differences are exact.
-__device__ inline void split3(const f32x2& x, bf16x2& h, bf16x2& m, bf16x2& l) {
-  h = __builtin_convertvector(x, bf16x2);
-  const f32x2 r1 = x - widen(h);
-  m = __builtin_convertvector(r1, bf16x2);
-  const f32x2 r2 = r1 - widen(m);
-  l = __builtin_convertvector(r2, bf16x2);
-}
-__device__ inline void split3(const f32x4& x, bf16x4& h, bf16x4& m, bf16x4& l) {
-  bf16x2 h0, m0, l0, h1, m1, l1;
-  split3(f32x2{x[0], x[1]}, h0, m0, l0);
-  split3(f32x2{x[2], x[3]}, h1, m1, l1);
-  h = __builtin_shufflevector(h0, h1, 0, 1, 2, 3);
-  m = __builtin_shufflevector(m0, m1, 0, 1, 2, 3);
-  l = __builtin_shufflevector(l0, l1, 0, 1, 2, 3);
-}
-__device__ inline bf16x8 cat8(const bf16x4& a, const bf16x4& b) {
-  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-__device__ inline float bf16_bits_to_float(unsigned short u) {
-  return __uint_as_float((unsigned)u << 16);
-}
-
 constexpr int XB_ROWS = 32;
 constexpr int XB_LDX = 272;                  // bytes per row of an X plane
 constexpr int XB_PLANE = XB_ROWS * XB_LDX;
@@ -1307,7 +1273,6 @@ constexpr int XB_RAW = XB_ROWS * XB_LDR * 4;
 constexpr int XB_LDS = XB_SLOT + 3 * XB_OPLANE + XB_RAW;
 constexpr int XB_FLUSH = 1024;               // tiles between flushes: 32,768 rows
 
-#define DN_MFMA_B16(A, B, C) __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, C, 0, 0, 0)
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_xg_mu_gram_b16(const float* __restrict__ X, const float* __restrict__ G, const float* num,
@@ -1521,12 +1486,6 @@ static int64_t xgg_parts(int64_t rows, int tile_rows, int flush, bool runs_of_ti
   if (wgs_out) *wgs_out = wgs;
   if (n_flush_out) *n_flush_out = n_flush;
   return wgs * n_flush;
-}
-
-// The bf16-split kernel is the default; DNPEFF_SPLIT_BF16=0 selects the fp32 matrix-core one.
-static bool use_split_bf16() {
-  const char* e = getenv("DNPEFF_SPLIT_BF16");
-  return e ? atoi(e) != 0 : true;
 }
 
 // Workspace of the fused update in floats, for `rows` rows.

@@ -115,6 +115,13 @@ int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials);
 int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr);
 
+// Products of the large matrix-core kernels run on the bf16 matrix cores with every fp32 operand
+// split in three (split_bf16.hpp) unless DNPEFF_SPLIT_BF16=0 selects the fp32 matrix cores.
+inline bool use_split_bf16() {
+  const char* e = getenv("DNPEFF_SPLIT_BF16");
+  return e ? atoi(e) != 0 : true;
+}
+
 // Columns present in many rows, held as a dense block in both orientations (head.hip).
 struct dense_head {
   int64_t n_d = 0;      // columns in the head

@@ -10,6 +10,7 @@
 // index K as their slow index: P = D^T ("cm", K = n_d) for the first, P = D ("rm", K = n) for
 // the second.
 #include "dnpeff_internal.hpp"
+#include "split_bf16.hpp"
 
 
 namespace dn {
@@ -201,6 +202,205 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
 }
 
 // ---------------------------------------------------------------------------
+// C[slice] = A[:, k in slice] B[:, k in slice]^T on the bf16 matrix cores, at fp32 accuracy.
+//
+// Both operands have the contraction index as their FAST index (A [M_pad, lda], B [N, ldb]): a
+// lane of v_mfma_f32_32x32x16_bf16 holds 8 consecutive contraction elements of one row, which
+// is then one 16-byte LDS read.  Every fp32 element is split in three bf16 parts once, on its
+// way into LDS (three planes per operand, rows of 32 elements padded to 80 bytes: conflict-free
+// 16-byte reads), and a product is six MFMAs (split_bf16.hpp).  A workgroup of 4 waves owns a
+// 128 x 128 tile of C (wave (wm, wn): 64 x 64) and one slice of the contraction tiles of 32,
+// dealt round-robin; the next tile travels in registers while the MFMAs of the current one run.
+// Per contraction tile a wave issues 48 MFMAs of 32 cycles and splits 32 elements (176 vector
+// instructions): 2240 SIMD cycles against 4096 for the 64 v_mfma_f32_32x32x2f32 of k_ptq.
+// Operands are zero-padded to whole tiles (rows to M_pad / N, the contraction to a multiple of
+// 32 within lda / ldb), so the loads need no bounds.
+// ---------------------------------------------------------------------------
+constexpr int ABT_KB = 32;
+constexpr int ABT_LD = 80;                // bytes per row of a plane
+constexpr int ABT_PLANE = 128 * ABT_LD;   // one part of one operand tile
+constexpr int ABT_LDS = 6 * ABT_PLANE;    // A: h, m, l; B: h, m, l
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_abt_b16(const float* __restrict__ A, int64_t lda, const float* __restrict__ B, int64_t ldb,
+              int64_t K, int N, int64_t M, int64_t M_pad, float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char ab[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t m0 = (int64_t)blockIdx.x * 128;
+  const int n0 = blockIdx.y * 128;
+  const int64_t k_tiles = (K + ABT_KB - 1) / ABT_KB;
+  const int64_t S = gridDim.z, z = blockIdx.z;
+  const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
+
+  // a thread fetches 16 bytes of 4 rows (32 rows apart) of each operand: 8 threads per row
+  const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
+  const float* a_src = A + (m0 + fr) * lda + fk;
+  const float* b_src = B + (int64_t)(n0 + fr) * ldb + fk;
+  f32x4 ra[4], rb[4];
+  auto fetch = [&](int64_t t) {
+    const int64_t k0 = (z + t * S) * ABT_KB;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      ra[q] = *reinterpret_cast<const f32x4*>(a_src + (int64_t)(32 * q) * lda + k0);
+      rb[q] = *reinterpret_cast<const f32x4*>(b_src + (int64_t)(32 * q) * ldb + k0);
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      bf16x4 h, m, l;
+      unsigned char* dst = ab + (fr + 32 * q) * ABT_LD + 2 * fk;
+      split3(ra[q], h, m, l);
+      *reinterpret_cast<bf16x4*>(dst) = h;
+      *reinterpret_cast<bf16x4*>(dst + ABT_PLANE) = m;
+      *reinterpret_cast<bf16x4*>(dst + 2 * ABT_PLANE) = l;
+      split3(rb[q], h, m, l);
+      *reinterpret_cast<bf16x4*>(dst + 3 * ABT_PLANE) = h;
+      *reinterpret_cast<bf16x4*>(dst + 4 * ABT_PLANE) = m;
+      *reinterpret_cast<bf16x4*>(dst + 5 * ABT_PLANE) = l;
+    }
+  };
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+  if (n_my > 0) {
+    fetch(0);
+    commit();
+  }
+  __syncthreads();
+  const unsigned char* a_row = ab + (64 * wm + l32) * ABT_LD + 16 * half;
+  const unsigned char* b_row = ab + 3 * ABT_PLANE + (64 * wn + l32) * ABT_LD + 16 * half;
+  for (int64_t t = 0; t < n_my; t++) {
+    if (t + 1 < n_my) fetch(t + 1);
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+      bf16x8 ah[2], am[2], al[2], bh[2], bm[2], bl[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const unsigned char* pa = a_row + 32 * i * ABT_LD + 32 * st;
+        ah[i] = *reinterpret_cast<const bf16x8*>(pa);
+        am[i] = *reinterpret_cast<const bf16x8*>(pa + ABT_PLANE);
+        al[i] = *reinterpret_cast<const bf16x8*>(pa + 2 * ABT_PLANE);
+        const unsigned char* pb = b_row + 32 * i * ABT_LD + 32 * st;
+        bh[i] = *reinterpret_cast<const bf16x8*>(pb);
+        bm[i] = *reinterpret_cast<const bf16x8*>(pb + ABT_PLANE);
+        bl[i] = *reinterpret_cast<const bf16x8*>(pb + 2 * ABT_PLANE);
+      }
+      // term by term over the four blocks: no instruction waits for the one before it
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bm[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bl[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(al[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bm[j], acc[i][j]);
+    }
+    __syncthreads();  // every wave is done with the planes
+    if (t + 1 < n_my) commit();
+    __syncthreads();
+  }
+
+  // D layout of a 32x32 block: reg v of lane l holds row 8 (v/4) + 4 (l/32) + v%4, column l%32;
+  // block (i, j) of the wave covers rows 64 wm + 32 i.., columns 64 wn + 32 j.. of the tile.
+  float* base = out + ((int64_t)blockIdx.z * M_pad + m0 + 64 * wm + 4 * half) * N + n0 + 64 * wn + l32;
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int below = 32 * i + 8 * (v >> 2) + (v & 3);
+        if (m0 + 64 * wm + 4 * half + below < M) base[(int64_t)below * N + 32 * j] = acc[i][j][v];
+      }
+}
+
+static int launch_abt_b16(const float* A, int64_t lda, const float* B, int64_t ldb, int64_t K, int N,
+                          int64_t M, int64_t M_pad, int64_t slices, float* out) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_abt_b16),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+    attr_set = true;
+  }
+  const int64_t k_pad = ceil_div(K, ABT_KB) * ABT_KB;
+  DN_CHECK(M_pad % 128 == 0 && N % 128 == 0 && lda % 4 == 0 && ldb % 4 == 0 && k_pad <= lda &&
+               k_pad <= ldb && ((uintptr_t)A % 16) == 0 && ((uintptr_t)B % 16) == 0,
+           "dense product: misaligned or unpadded operands");
+  DN_CHECK(M_pad / 128 < ((int64_t)1 << 22), "dense product: too many row tiles");
+  dim3 grid((unsigned)(M_pad / 128), (unsigned)(N / 128), (unsigned)slices);
+  hipLaunchKernelGGL(k_abt_b16, grid, dim3(256), ABT_LDS, stream(), A, lda, B, ldb, K, N, M, M_pad, out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+// out[c * ld + i] = in[i * cols + c] for i < rows, 0 for rows <= i < ld   (32 x 32 tiles via LDS)
+__global__ void __launch_bounds__(256)
+    k_transpose_pad(const float* __restrict__ in, int64_t rows, int cols, int64_t ld,
+                    float* __restrict__ out) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t i0 = (int64_t)blockIdx.x * 32;
+  const int c0 = blockIdx.y * 32;
+  for (int q = ty; q < 32; q += 8) {
+    const int64_t i = i0 + q;
+    const int c = c0 + tx;
+    tile[q][tx] = (i < rows && c < cols) ? in[i * cols + c] : 0.0f;
+  }
+  __syncthreads();
+  for (int q = ty; q < 32; q += 8) {
+    const int c = c0 + q;
+    const int64_t i = i0 + tx;
+    if (c < cols && i < ld) out[(int64_t)c * ld + i] = tile[tx][q];
+  }
+}
+
+// out[j * ld + k] = H[cols[k]][j] for k < n_d, 0 for n_d <= k < ld
+__global__ void __launch_bounds__(256)
+    k_head_gather_t(const float* __restrict__ H, const int32_t* __restrict__ cols, int64_t n_d, int r,
+                    int64_t ld, float* __restrict__ out) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t k0 = (int64_t)blockIdx.x * 32;
+  const int j0 = blockIdx.y * 32;
+  for (int q = ty; q < 32; q += 8) {
+    const int64_t k = k0 + q;
+    const int j = j0 + tx;
+    tile[q][tx] = (k < n_d && j < r) ? H[(int64_t)cols[k] * r + j] : 0.0f;
+  }
+  __syncthreads();
+  for (int q = ty; q < 32; q += 8) {
+    const int j = j0 + q;
+    const int64_t k = k0 + tx;
+    if (j < r && k < ld) out[(int64_t)j * ld + k] = tile[tx][q];
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Gram X^T X for ranks that are multiples of 128 above 128: the same tiles with P = Q = X, only
 // the tile pairs (i <= j), K split into slices; the reduction sums the slices in fp64 and writes
 // every element and its mirror image.
@@ -308,6 +508,13 @@ static unsigned elem_grid(int64_t count) {
   return (unsigned)(g < 1 ? 1 : g);
 }
 
+// At ranks that are multiples of 128 the head products run on the bf16 matrix cores with split
+// operands (k_abt_b16), otherwise (and with DNPEFF_SPLIT_BF16=0) on the fp32 ones (k_ptq).
+static bool head_uses_split(int r) { return r % 128 == 0 && use_split_bf16(); }
+static int64_t head_gather_floats(const dense_head& h, int r) {
+  return (h.n_d_pad > h.n_pad ? h.n_d_pad : h.n_pad) * (int64_t)r;
+}
+
 static int64_t head_slices_n(const dense_head& h, int r) {
   return ptq_slices((h.n_pad / 128) * ceil_div(r, 128), ceil_div(h.n_d, PTQ_KB));
 }
@@ -319,7 +526,9 @@ int head_ensure_workspace(dnpeff_csr* A, int r) {
   dense_head& h = A->head;
   if (h.n_d == 0) return 0;
   DN_CHECK(r % 4 == 0, "a matrix with a dense head needs a rank that is a multiple of 4 (got %d)", r);
-  const int64_t gather = h.n_d_pad * r;
+  // gathered rows of H of the head, or W transposed (the split-operand product wants the
+  // contraction index fast)
+  const int64_t gather = head_gather_floats(h, r);
   const int64_t wn = head_slices_n(h, r) * h.n_pad * r;
   const int64_t wt = head_slices_t(h, r, A->n_rows) * h.n_d_pad * r;
   const int64_t need = gather + (wn > wt ? wn : wt);
@@ -337,7 +546,14 @@ int launch_head_n(const dnpeff_csr* A, int r, const float* H_mr) {
   if (h.n_d == 0) return 0;
   DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)H_mr % 16) == 0, "dense head: workspace or alignment");
   float* Hd = h.ws;
-  float* part = h.ws + h.n_d_pad * r;
+  float* part = h.ws + head_gather_floats(h, r);
+  if (head_uses_split(r)) {
+    // D [n, n_d] (rm) times the gathered rows, transposed: contraction over the head slots
+    dim3 tg((unsigned)ceil_div(h.n_d_pad, 32), (unsigned)ceil_div(r, 32));
+    hipLaunchKernelGGL(k_head_gather_t, tg, dim3(256), 0, stream(), H_mr, h.cols, h.n_d, r, h.n_d_pad, Hd);
+    return launch_abt_b16(h.rm, h.n_d_pad, Hd, h.n_d_pad, h.n_d, r, A->n_rows, h.n_pad,
+                          head_slices_n(h, r), part);
+  }
   hipLaunchKernelGGL(k_head_gather, dim3(elem_grid(h.n_d * (r / 4))), dim3(256), 0, stream(), H_mr,
                      h.cols, h.n_d, r, Hd);
   return launch_ptq(h.cm, h.n_pad, h.n_d, Hd, r, A->n_rows, h.n_pad, head_slices_n(h, r), part);
@@ -347,7 +563,7 @@ int launch_head_n(const dnpeff_csr* A, int r, const float* H_mr) {
 int launch_head_n_add(const dnpeff_csr* A, int r, float* N_nr) {
   const dense_head& h = A->head;
   if (h.n_d == 0) return 0;
-  const float* part = h.ws + h.n_d_pad * r;
+  const float* part = h.ws + head_gather_floats(h, r);
   hipLaunchKernelGGL(k_head_add, dim3(elem_grid(A->n_rows * (r / 4))), dim3(256), 0, stream(), part,
                      head_slices_n(h, r), A->n_rows, h.n_pad, r, N_nr);
   DN_LAUNCH_CHECK();
@@ -360,9 +576,17 @@ int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
   if (h.n_d == 0) return 0;
   DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)W_nr % 16) == 0 && ((uintptr_t)T_mr % 16) == 0,
            "dense head: workspace or alignment");
-  float* part = h.ws + h.n_d_pad * r;
+  float* part = h.ws + head_gather_floats(h, r);
   const int64_t slices = head_slices_t(h, r, A->n_rows);
-  DN_TRY(launch_ptq(h.rm, h.n_d_pad, A->n_rows, W_nr, r, h.n_d, h.n_d_pad, slices, part));
+  if (head_uses_split(r)) {
+    // D^T [n_d, n] (cm) times W transposed: contraction over the rows of the matrix
+    float* Wt = h.ws;
+    dim3 tg((unsigned)ceil_div(h.n_pad, 32), (unsigned)ceil_div(r, 32));
+    hipLaunchKernelGGL(k_transpose_pad, tg, dim3(256), 0, stream(), W_nr, A->n_rows, r, h.n_pad, Wt);
+    DN_TRY(launch_abt_b16(h.cm, h.n_pad, Wt, h.n_pad, A->n_rows, r, h.n_d, h.n_d_pad, slices, part));
+  } else {
+    DN_TRY(launch_ptq(h.rm, h.n_d_pad, A->n_rows, W_nr, r, h.n_d, h.n_d_pad, slices, part));
+  }
   hipLaunchKernelGGL(k_head_scatter, dim3(elem_grid(h.n_d * (r / 4))), dim3(256), 0, stream(), part,
                      slices, h.n_d, h.n_d_pad, r, h.cols, T_mr);
   DN_LAUNCH_CHECK();
