@@ -1,0 +1,136 @@
+// Main loop of the split-operand matrix products: C (128 x 128 per workgroup) +=
+// A (128 x K) B (128 x K)^T on the bf16 matrix cores at fp32 accuracy (split_bf16.hpp).
+#pragma once
+#include "split_bf16.hpp"
+
+namespace dn {
+
+typedef float abt_acc16 __attribute__((ext_vector_type(16)));
+
+constexpr int ABT_KB = 32;
+constexpr int ABT_LD = 80;                // bytes per row of a plane: 32 bf16 + 16 of padding
+constexpr int ABT_PLANE = 128 * ABT_LD;   // one part of one operand tile
+constexpr int ABT_LDS = 6 * ABT_PLANE;    // A: h, m, l; B: h, m, l
+
+// One operand tile (128 rows x 32 contraction elements) on its way from global memory to the
+// three bf16 planes in LDS.  KN = false: the source has the contraction index fast
+// (src[row * ld + k]): a thread takes 16 bytes of 4 rows, 8 threads per row.  KN = true: the
+// source has it slow (src[k * ld + row], e.g. a tile of X for X^T X): a thread takes 16
+// contraction elements of one row with 4-byte loads that are coalesced across the lanes, and
+// four consecutive ones make one 8-byte LDS store either way.
+template <bool KN>
+struct AbtOperand {
+  f32x4 r[4];
+  __device__ __forceinline__ void fetch(const float* __restrict__ src, int64_t ld, int64_t k0) {
+    if constexpr (!KN) {
+      const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        r[q] = *reinterpret_cast<const f32x4*>(src + (int64_t)(fr + 32 * q) * ld + k0 + fk);
+    } else {
+      const int row = threadIdx.x & 127, kq = threadIdx.x >> 7;
+      const float* p = src + (k0 + 16 * kq) * ld + row;
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int u = 0; u < 4; u++) r[q][u] = p[(int64_t)(4 * q + u) * ld];
+    }
+  }
+  __device__ __forceinline__ void commit(unsigned char* planes) const {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      bf16x4 h, m, l;
+      split3(r[q], h, m, l);
+      unsigned char* dst;
+      if constexpr (!KN) {
+        const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
+        dst = planes + (fr + 32 * q) * ABT_LD + 2 * fk;
+      } else {
+        const int row = threadIdx.x & 127, kq = threadIdx.x >> 7;
+        dst = planes + row * ABT_LD + 2 * (16 * kq + 4 * q);
+      }
+      *reinterpret_cast<bf16x4*>(dst) = h;
+      *reinterpret_cast<bf16x4*>(dst + ABT_PLANE) = m;
+      *reinterpret_cast<bf16x4*>(dst + 2 * ABT_PLANE) = l;
+    }
+  }
+};
+
+// acc += A B^T over the contraction tiles first, first + stride, ... (n_tiles of them).  Wave
+// (wm, wn) of the four owns the 64 x 64 quarter of the tile: blocks (i, j) of 32 x 32.  The next
+// contraction tile travels in registers while the 48 MFMAs of the current one run; every fp32
+// element is split once, on its way into LDS.  The sources must be readable for whole tiles
+// (zero padding, or rows clamped by the caller's pointer arithmetic).
+template <bool A_KN, bool B_KN>
+__device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, int64_t lda,
+                                             const float* __restrict__ b_src, int64_t ldb,
+                                             int64_t first, int64_t stride, int64_t n_tiles,
+                                             unsigned char* ab, abt_acc16 (&acc)[2][2]) {
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l32 = lane & 31, half = lane >> 5, wm = wave >> 1, wn = wave & 1;
+  AbtOperand<A_KN> oa;
+  AbtOperand<B_KN> ob;
+  if (n_tiles > 0) {
+    oa.fetch(a_src, lda, first * ABT_KB);
+    ob.fetch(b_src, ldb, first * ABT_KB);
+    oa.commit(ab);
+    ob.commit(ab + 3 * ABT_PLANE);
+  }
+  __syncthreads();
+  const unsigned char* a_row = ab + (64 * wm + l32) * ABT_LD + 16 * half;
+  const unsigned char* b_row = ab + 3 * ABT_PLANE + (64 * wn + l32) * ABT_LD + 16 * half;
+  for (int64_t t = 0; t < n_tiles; t++) {
+    if (t + 1 < n_tiles) {
+      oa.fetch(a_src, lda, (first + (t + 1) * stride) * ABT_KB);
+      ob.fetch(b_src, ldb, (first + (t + 1) * stride) * ABT_KB);
+    }
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+      bf16x8 ah[2], am[2], al[2], bh[2], bm[2], bl[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const unsigned char* pa = a_row + 32 * i * ABT_LD + 32 * st;
+        ah[i] = *reinterpret_cast<const bf16x8*>(pa);
+        am[i] = *reinterpret_cast<const bf16x8*>(pa + ABT_PLANE);
+        al[i] = *reinterpret_cast<const bf16x8*>(pa + 2 * ABT_PLANE);
+        const unsigned char* pb = b_row + 32 * i * ABT_LD + 32 * st;
+        bh[i] = *reinterpret_cast<const bf16x8*>(pb);
+        bm[i] = *reinterpret_cast<const bf16x8*>(pb + ABT_PLANE);
+        bl[i] = *reinterpret_cast<const bf16x8*>(pb + 2 * ABT_PLANE);
+      }
+      // term by term over the four blocks: no instruction waits for the one before it
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bm[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bl[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(al[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bm[j], acc[i][j]);
+    }
+    __syncthreads();  // every wave is done with the planes
+    if (t + 1 < n_tiles) {
+      oa.commit(ab);
+      ob.commit(ab + 3 * ABT_PLANE);
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace dn

@@ -3,7 +3,7 @@
 // multiplicative update fused into the X G epilogue, dot products with fp64
 // accumulation, seeded initialisation and the [m, r] <-> [r, m] transposition.
 #include "dnpeff_internal.hpp"
-#include "split_bf16.hpp"
+#include "abt_b16.hpp"
 #include "synth_rng.h"
 
 #include <type_traits>
@@ -978,6 +978,122 @@ static int launch_xg_mu_tile(int64_t rows, int r, const float* X, const float* G
   return 0;
 }
 
+// The same update on the bf16 matrix cores with split operands (abt_b16.hpp): X has the
+// contraction index fast as it is, G is passed transposed (Gt[n][k] = G[k][n]).  Whole row tiles
+// of 128 only; the caller hands the last rows to k_xg_mu_tile.
+template <bool WITH_D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_xg_mu_tile_b16(const float* __restrict__ X, const float* __restrict__ Gt, const float* num,
+                     float eps, int64_t n_row_tiles, int r, int n_chunks, float* out,
+                     float* __restrict__ D_out) {
+  extern __shared__ __align__(16) unsigned char ab[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  // Workgroups are dealt to the 8 XCDs round-robin by their number; the column chunks of one row
+  // tile are numbered 8 apart so that they share an XCD, i.e. an L2, and X comes in once.
+  const int64_t grp = blockIdx.x / (8 * n_chunks);
+  const int rem = (int)(blockIdx.x % (8 * n_chunks));
+  const int64_t tile = grp * 8 + rem % 8;
+  if (tile >= n_row_tiles) return;
+  const int n0 = (rem / 8) * 128;
+  const int64_t row0 = tile * 128;
+
+  // element (i, j, v): row 64 wm + 32 i + 8 (v / 4) + 4 half + v % 4, column n0 + 64 wn + 32 j + l32
+  const int64_t t0 = (row0 + 64 * wm + 4 * half) * (int64_t)r + n0 + 64 * wn;
+  const float* tnum = num + t0;
+  const float* tx = X + t0;
+  float* tout = out + t0;
+  float* tD = WITH_D ? D_out + t0 : nullptr;
+  float pn[2][16], px[2][16];
+  auto request = [&](int blk, float (&n_)[16], float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int64_t off = (32 * i + 8 * (v >> 2) + (v & 3)) * (int64_t)r + 32 * j + l32;
+      n_[v] = tnum[off];
+      x_[v] = tx[off];
+    }
+  };
+  // the epilogue operands of the first block are requested before the contraction starts
+  request(0, pn[0], px[0]);
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+  abt_mainloop<false, false>(X + row0 * r, r, Gt + (int64_t)n0 * r, r, 0, 1, r / ABT_KB, ab, acc);
+
+  auto finish = [&](int blk, const float (&n_)[16], const float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int64_t off = (32 * i + 8 * (v >> 2) + (v & 3)) * (int64_t)r + 32 * j + l32;
+      const float d = acc[i][j][v];
+      const float q = n_[v] / (d + eps);
+      tout[off] = x_[v] * q;
+      if (WITH_D) tD[off] = d;
+    }
+  };
+  request(1, pn[1], px[1]);
+  finish(0, pn[0], px[0]);
+  request(2, pn[0], px[0]);
+  finish(1, pn[1], px[1]);
+  request(3, pn[1], px[1]);
+  finish(2, pn[0], px[0]);
+  finish(3, pn[1], px[1]);
+}
+
+// G transposed for the split-operand update: a buffer that grows to the largest rank seen and
+// lives until the process ends (one host thread drives the library).
+static float* g_gt = nullptr;
+static int64_t g_gt_floats = 0;
+
+static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const float* G, const float* num,
+                                 float eps, float* out, float* D_out) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_tile_b16<false>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+    DN_HIP(hipFuncSetAttribute((const void*)k_xg_mu_tile_b16<true>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+    attr_set = true;
+  }
+  if (g_gt_floats < (int64_t)r * r) {
+    DN_HIP(hipStreamSynchronize(stream()));
+    dfree(g_gt);
+    g_gt = nullptr;
+    g_gt_floats = 0;
+    DN_TRY(dmalloc(&g_gt, (int64_t)r * r));
+    g_gt_floats = (int64_t)r * r;
+  }
+  DN_TRY(launch_transpose(r, r, G, g_gt));
+  const int n_chunks = r / 128;
+  const int64_t tiles = rows / 128;
+  if (tiles > 0) {
+    const int64_t wgs = ceil_div(tiles, 8) * 8 * n_chunks;
+    DN_CHECK(wgs < ((int64_t)1 << 24), "xg_mu: too many tiles for one launch");
+    const dim3 grid((unsigned)wgs), block(256);
+    if (D_out)
+      hipLaunchKernelGGL((k_xg_mu_tile_b16<true>), grid, block, ABT_LDS, stream(), X, g_gt, num, eps,
+                         tiles, r, n_chunks, out, D_out);
+    else
+      hipLaunchKernelGGL((k_xg_mu_tile_b16<false>), grid, block, ABT_LDS, stream(), X, g_gt, num, eps,
+                         tiles, r, n_chunks, out, D_out);
+    DN_LAUNCH_CHECK();
+  }
+  const int64_t head = tiles * 128;
+  if (head < rows) {
+    const int64_t off = head * r;
+    DN_TRY(launch_xg_mu_tile(rows - head, r, X + off, G, num + off, eps, out + off,
+                             D_out ? D_out + off : nullptr));
+  }
+  return 0;
+}
+
 template <int NB, int PD, bool VEC4>
 static int launch_xg_mu_inst(dim3 grid, size_t lds, const float* X, const float* G,
                              const float* num, float eps, int64_t rows, int r, int nsteps,
@@ -1586,8 +1702,11 @@ int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const floa
                               D_out ? D_out + off : nullptr);
   }
   if (r > 128 && r % 128 == 0 && aligned && ((uintptr_t)G % 16) == 0 && rows >= 256 &&
-      ceil_div(rows, 128) * (r / 128) < ((int64_t)1 << 24))
+      ceil_div(rows, 128) * (r / 128) < ((int64_t)1 << 24)) {
+    if (use_split_bf16() && ((uintptr_t)num % 4) == 0)
+      return launch_xg_mu_tile_b16(rows, r, X, G, num, eps, out, D_out);
     return launch_xg_mu_tile(rows, r, X, G, num, eps, out, D_out);
+  }
   // widest column chunk whose slice of G fits 128 KB of LDS
   if (r <= 256) return launch_xg_mu_nb<4>(rows, r, X, G, num, eps, out, D_out);
   if (r <= 512) return launch_xg_mu_nb<2>(rows, r, X, G, num, eps, out, D_out);

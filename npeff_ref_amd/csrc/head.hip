@@ -10,7 +10,7 @@
 // index K as their slow index: P = D^T ("cm", K = n_d) for the first, P = D ("rm", K = n) for
 // the second.
 #include "dnpeff_internal.hpp"
-#include "split_bf16.hpp"
+#include "abt_b16.hpp"
 
 
 namespace dn {
@@ -216,11 +216,6 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
 // Operands are zero-padded to whole tiles (rows to M_pad / N, the contraction to a multiple of
 // 32 within lda / ldb), so the loads need no bounds.
 // ---------------------------------------------------------------------------
-constexpr int ABT_KB = 32;
-constexpr int ABT_LD = 80;                // bytes per row of a plane
-constexpr int ABT_PLANE = 128 * ABT_LD;   // one part of one operand tile
-constexpr int ABT_LDS = 6 * ABT_PLANE;    // A: h, m, l; B: h, m, l
-
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_abt_b16(const float* __restrict__ A, int64_t lda, const float* __restrict__ B, int64_t ldb,
               int64_t K, int N, int64_t M, int64_t M_pad, float* __restrict__ out) {
@@ -234,35 +229,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int64_t S = gridDim.z, z = blockIdx.z;
   const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
 
-  // a thread fetches 16 bytes of 4 rows (32 rows apart) of each operand: 8 threads per row
-  const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
-  const float* a_src = A + (m0 + fr) * lda + fk;
-  const float* b_src = B + (int64_t)(n0 + fr) * ldb + fk;
-  f32x4 ra[4], rb[4];
-  auto fetch = [&](int64_t t) {
-    const int64_t k0 = (z + t * S) * ABT_KB;
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-      ra[q] = *reinterpret_cast<const f32x4*>(a_src + (int64_t)(32 * q) * lda + k0);
-      rb[q] = *reinterpret_cast<const f32x4*>(b_src + (int64_t)(32 * q) * ldb + k0);
-    }
-  };
-  auto commit = [&]() {
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-      bf16x4 h, m, l;
-      unsigned char* dst = ab + (fr + 32 * q) * ABT_LD + 2 * fk;
-      split3(ra[q], h, m, l);
-      *reinterpret_cast<bf16x4*>(dst) = h;
-      *reinterpret_cast<bf16x4*>(dst + ABT_PLANE) = m;
-      *reinterpret_cast<bf16x4*>(dst + 2 * ABT_PLANE) = l;
-      split3(rb[q], h, m, l);
-      *reinterpret_cast<bf16x4*>(dst + 3 * ABT_PLANE) = h;
-      *reinterpret_cast<bf16x4*>(dst + 4 * ABT_PLANE) = m;
-      *reinterpret_cast<bf16x4*>(dst + 5 * ABT_PLANE) = l;
-    }
-  };
-
   acc16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
@@ -270,60 +236,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-
-  if (n_my > 0) {
-    fetch(0);
-    commit();
-  }
-  __syncthreads();
-  const unsigned char* a_row = ab + (64 * wm + l32) * ABT_LD + 16 * half;
-  const unsigned char* b_row = ab + 3 * ABT_PLANE + (64 * wn + l32) * ABT_LD + 16 * half;
-  for (int64_t t = 0; t < n_my; t++) {
-    if (t + 1 < n_my) fetch(t + 1);
-#pragma unroll
-    for (int st = 0; st < 2; st++) {
-      bf16x8 ah[2], am[2], al[2], bh[2], bm[2], bl[2];
-#pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const unsigned char* pa = a_row + 32 * i * ABT_LD + 32 * st;
-        ah[i] = *reinterpret_cast<const bf16x8*>(pa);
-        am[i] = *reinterpret_cast<const bf16x8*>(pa + ABT_PLANE);
-        al[i] = *reinterpret_cast<const bf16x8*>(pa + 2 * ABT_PLANE);
-        const unsigned char* pb = b_row + 32 * i * ABT_LD + 32 * st;
-        bh[i] = *reinterpret_cast<const bf16x8*>(pb);
-        bm[i] = *reinterpret_cast<const bf16x8*>(pb + ABT_PLANE);
-        bl[i] = *reinterpret_cast<const bf16x8*>(pb + 2 * ABT_PLANE);
-      }
-      // term by term over the four blocks: no instruction waits for the one before it
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bh[j], acc[i][j]);
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bm[j], acc[i][j]);
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bh[j], acc[i][j]);
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bl[j], acc[i][j]);
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(al[i], bh[j], acc[i][j]);
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bm[j], acc[i][j]);
-    }
-    __syncthreads();  // every wave is done with the planes
-    if (t + 1 < n_my) commit();
-    __syncthreads();
-  }
+  abt_mainloop<false, false>(A + m0 * lda, lda, B + (int64_t)n0 * ldb, ldb, z, S, n_my, ab, acc);
 
   // D layout of a 32x32 block: reg v of lane l holds row 8 (v/4) + 4 (l/32) + v%4, column l%32;
   // block (i, j) of the wave covers rows 64 wm + 32 i.., columns 64 wn + 32 j.. of the tile.
@@ -415,7 +328,7 @@ static int64_t gram_tiles_slices(int64_t rows, int r) {
 }
 
 int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
-  return gram_tiles_slices(rows, r) * (int64_t)r * r;
+  return (gram_tiles_slices(rows, r) + 1) * (int64_t)r * r;
 }
 
 __global__ void __launch_bounds__(256)
@@ -431,9 +344,72 @@ __global__ void __launch_bounds__(256)
   G[(int64_t)b * r + a] = (float)s;
 }
 
+// The same on the bf16 matrix cores with split operands (abt_b16.hpp): both operand tiles are
+// column tiles of X, read with the contraction index (the rows of X) slow.  Whole contraction
+// tiles of 32 rows only; the caller adds the last rows.
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_gram_tiles_b16(const float* __restrict__ X, int64_t k_tiles, int r, int n_tiles_side,
+                     float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char ab[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  // grid.x numbers the tile pairs (ti <= tj) row by row: every workgroup of the grid works
+  int p = blockIdx.x, row_len = n_tiles_side, ti = 0;
+  while (p >= row_len) {
+    p -= row_len;
+    ti++;
+    row_len--;
+  }
+  const int tj = ti + p;
+  const int64_t S = gridDim.z, z = blockIdx.z;
+  const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+  abt_mainloop<true, true>(X + 128 * ti, r, X + 128 * tj, r, z, S, n_my, ab, acc);
+  float* base = out + ((int64_t)z * r + 128 * ti + 64 * wm + 4 * half) * r + 128 * tj + 64 * wn + l32;
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        base[(int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * r + 32 * j] = acc[i][j][v];
+}
+
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace) {
-  const int64_t slices = gram_tiles_slices(rows, r);
-  DN_TRY(launch_ptq(X, r, rows, X, r, r, r, slices, workspace, r / 128));
+  int64_t slices = gram_tiles_slices(rows, r);
+  const int t = r / 128;
+  if (use_split_bf16() && rows >= ABT_KB) {
+    static bool attr_set = false;
+    if (!attr_set) {
+      DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_tiles_b16),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+      attr_set = true;
+    }
+    // whole contraction tiles on the bf16 matrix cores, the last rows (fewer than 32) as one
+    // more slice through the fp32 kernel
+    const int64_t k_tiles = rows / ABT_KB, whole = k_tiles * ABT_KB;
+    int64_t s = slices - 1;
+    if (s < 1) s = 1;
+    if (s > k_tiles) s = k_tiles;
+    hipLaunchKernelGGL(k_gram_tiles_b16, dim3((unsigned)(t * (t + 1) / 2), 1, (unsigned)s), dim3(256),
+                       ABT_LDS, stream(), X, k_tiles, r, t, workspace);
+    DN_LAUNCH_CHECK();
+    slices = s;
+    if (whole < rows) {
+      DN_TRY(launch_ptq(X + whole * r, r, rows - whole, X + whole * r, r, r, r, 1,
+                        workspace + s * (int64_t)r * r, t));
+      slices = s + 1;
+    }
+  } else {
+    DN_TRY(launch_ptq(X, r, rows, X, r, r, r, slices, workspace, t));
+  }
   hipLaunchKernelGGL(k_gram_tiles_reduce, dim3((unsigned)ceil_div((int64_t)r * r, 256)), dim3(256), 0,
                      stream(), workspace, slices, r, G);
   DN_LAUNCH_CHECK();
