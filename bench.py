@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
 MFMA_FP32_PEAK = 157.3e12  # flop/s, dense fp32 matrix
+MFMA_BF16_PEAK = 2.5e15  # flop/s, dense bf16 matrix
 
 CONFIGS = {
     "c0": dict(n=512, m_full=1 << 20, k=4096, kmin=0, kmax=0, s=1.1, r=16),
@@ -52,32 +53,47 @@ def log(msg):
 
 
 def algorithmic(cls, n, m, z, r, fused_gram=False, split_bf16=False):
-    """Compulsory traffic / flops of one launch: every operand touched once.  With fused_gram the
-    H update also produces H^T H (no separate gram_H launch): its class carries both products.
-    With split_bf16 those products run on the bf16 matrix cores (every fp32 operand as the sum of
-    three bf16 numbers, six partial products, fp32 accumulation), whose peak is 16 times the fp32
-    cores': the launch is then bounded by its three passes over m x r floats, not by arithmetic."""
+    """Compulsory work of one launch, every operand touched once: (bytes, fp32 flops, split).
+    flops = 0 for the kernels without a matrix product.  With fused_gram the H update also
+    produces H^T H (no separate gram_H launch): its class carries both products.  split = the
+    products run on the bf16 matrix cores (every fp32 operand as the sum of three bf16 numbers,
+    six partial products, fp32 accumulation): the launch then executes 6 x flops on a peak that
+    is 16 times the fp32 cores'."""
     P = 4 if z < 2**31 else 8
+    tiles = split_bf16 and r > 128 and r % 128 == 0  # the 128 x 128 tile kernels
     if cls == "spmm_n":
-        return "hbm", 8 * z + P * (n + 1) + 4 * r * m + 4 * n * r
+        return 8 * z + P * (n + 1) + 4 * r * m + 4 * n * r, 0, False
     if cls == "spmm_n_reduce":
-        return "hbm", 8 * n * r
+        return 8 * n * r, 0, False
     if cls == "spmm_t":
-        return "hbm", 8 * z + P * (m + 1) + 4 * n * r + 4 * r * m
+        return 8 * z + P * (m + 1) + 4 * n * r + 4 * r * m, 0, False
     # a Gram matrix is symmetric: r (r + 1) / 2 distinct dot products of length e
     if cls == "gram_H":
-        return ("mfma", m * r * (r + 1)) if r >= 64 else ("hbm", 4 * m * r + 4 * r * r)
+        return 4 * m * r + 4 * r * r, m * r * (r + 1), tiles and m >= 1024
     if cls == "gram_W":
-        return ("mfma", n * r * (r + 1)) if r >= 64 else ("hbm", 4 * n * r + 4 * r * r)
+        return 4 * n * r + 4 * r * r, n * r * (r + 1), tiles and n >= 1024
     if cls == "xg_mu_H":
-        if fused_gram and split_bf16:
-            return "hbm", 12 * m * r + 8 * r * r
         if fused_gram:
-            return "mfma", 2 * m * r * r + m * r * (r + 1)
-        return ("mfma", 2 * m * r * r) if r >= 64 else ("hbm", 12 * m * r + 4 * r * r)
+            return 12 * m * r + 8 * r * r, 2 * m * r * r + m * r * (r + 1), split_bf16
+        return 12 * m * r + 4 * r * r, 2 * m * r * r, tiles and m >= 256
     if cls == "xg_mu_W":
-        return ("mfma", 2 * n * r * r) if r >= 64 else ("hbm", 12 * n * r + 4 * r * r)
+        return 12 * n * r + 4 * r * r, 2 * n * r * r, tiles and n >= 256
     raise KeyError(cls)
+
+
+def price(cls, n, m, z, r, avg_s, fused_gram, split_bf16):
+    """The roofline that binds a launch of mean duration avg_s: the larger of its HBM fraction and
+    its matrix-core fraction (fp32 cores, or bf16 cores for the split-operand kernels)."""
+    nbytes, flops, split = algorithmic(cls, n, m, z, r, fused_gram, split_bf16)
+    f_hbm = nbytes / avg_s / HBM_PEAK
+    f_mm = (6 * flops / avg_s / MFMA_BF16_PEAK) if split else (flops / avg_s / MFMA_FP32_PEAK)
+    if f_mm > f_hbm:
+        done = 6 * flops if split else flops
+        return dict(bound="mfma", achieved=done / avg_s / 1e12, unit="TFLOP/s",
+                    peak=(MFMA_BF16_PEAK if split else MFMA_FP32_PEAK) / 1e12, frac=f_mm,
+                    arithmetic="bf16 x 6 (split fp32 operands)" if split else "fp32")
+    return dict(bound="hbm", achieved=nbytes / avg_s / 1e9, unit="GB/s", peak=HBM_PEAK / 1e9,
+                frac=f_hbm)
 
 
 def prepare_cpu_baseline(d, A, nmf, n, m, r, eps):
@@ -180,24 +196,18 @@ def main():
 
     kernels = {}
     fused_gram = tim.get("gram_H", (0.0, 0))[1] == 0
-    split_bf16 = fused_gram and os.environ.get("DNPEFF_SPLIT_BF16", "1") != "0"
+    split_bf16 = os.environ.get("DNPEFF_SPLIT_BF16", "1") != "0"
     for cls, (ms_sum, cnt) in tim.items():
         if cnt == 0:
             continue
-        bound, work = algorithmic(cls, n, m, z, r, fused_gram, split_bf16)
         avg_s = ms_sum / cnt * 1e-3
-        peak = HBM_PEAK if bound == "hbm" else MFMA_FP32_PEAK
-        kernels[cls] = dict(
-            ms=ms_sum / cnt, bound=bound,
-            achieved=work / avg_s / 1e9 if bound == "hbm" else work / avg_s / 1e12,
-            unit="GB/s" if bound == "hbm" else "TFLOP/s", frac=work / avg_s / peak,
-            share=ms_sum / (elapsed * 1e3))
-        k = kernels[cls]
+        k = price(cls, n, m, z, r, avg_s, fused_gram, split_bf16)
+        k.update(ms=ms_sum / cnt, share=ms_sum / (elapsed * 1e3))
+        kernels[cls] = k
         log(f"  {cls:14s} {k['ms']:9.3f} ms  {k['achieved']:9.1f} {k['unit']:8s} frac {k['frac']:.3f}")
     dom = max((k for k in kernels if k != "spmm_n_reduce"), key=lambda k: kernels[k]["ms"])
     kd = kernels[dom]
-    roofline = dict(kernel=dom, bound=kd["bound"], achieved=kd["achieved"],
-                    peak=HBM_PEAK / 1e9 if kd["bound"] == "hbm" else MFMA_FP32_PEAK / 1e12,
+    roofline = dict(kernel=dom, bound=kd["bound"], achieved=kd["achieved"], peak=kd["peak"],
                     unit=kd["unit"], frac=kd["frac"],
                     traffic=TRAFFIC_C1.get(dom) if args.config == "c1" else None)
 
@@ -225,8 +235,9 @@ def main():
         "cpu_baseline": cpu_baseline,
         "kernels": kernels,
         "fused_gram_in_H_update": fused_gram,
-        "h_update_products": ("bf16 MFMA on fp32 operands split in three (6 partial products, fp32 "
-                              "accumulation, fp32 accuracy)" if split_bf16 else "fp32 MFMA"),
+        "matrix_products": ("bf16 MFMA on fp32 operands split in three (6 partial products, fp32 "
+                            "accumulation, fp32 accuracy) where the kernel table says so"
+                            if split_bf16 else "fp32 MFMA"),
         "spmm_hbm_frac": {k: kernels[k]["frac"] for k in ("spmm_n", "spmm_t") if k in kernels},
         "loss_after": loss,
     }

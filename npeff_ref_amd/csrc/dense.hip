@@ -1015,9 +1015,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       x_[v] = tx[off];
     }
   };
-  // the epilogue operands of the first block are requested before the contraction starts
-  request(0, pn[0], px[0]);
-
   acc16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
@@ -1038,6 +1035,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       if (WITH_D) tD[off] = d;
     }
   };
+  request(0, pn[0], px[0]);
   request(1, pn[1], px[1]);
   finish(0, pn[0], px[0]);
   request(2, pn[0], px[0]);
