@@ -247,9 +247,14 @@ DN_API int dnpeff_nmf_loss_terms(dnpeff_nmf* h, double* sq_norm_A, double* pos, 
   DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
   DN_TRY(launch_dot(h->n * h->r, h->Nw, h->W, h->dot_ws, h->dot_ws + DOT_BLOCKS));
   // pos = <H, (W^T W) H> = <W^T W, H H^T>
-  DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
+  // (H^T H of the current H is at hand when the last H update produced it)
+  const float* Gh = h->G;
+  if (h->GH && h->gh_valid)
+    Gh = h->GH;
+  else
+    DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
   DN_TRY(launch_gram(h->n, h->r, h->W, h->G2, h->gram_ws));
-  DN_TRY(launch_dot((int64_t)h->r * h->r, h->G, h->G2, h->dot_ws, h->dot_ws + DOT_BLOCKS + 1));
+  DN_TRY(launch_dot((int64_t)h->r * h->r, Gh, h->G2, h->dot_ws, h->dot_ws + DOT_BLOCKS + 1));
   double res[2];
   DN_HIP(hipStreamSynchronize(stream()));
   DN_HIP(hipMemcpy(res, h->dot_ws + DOT_BLOCKS, sizeof(double) * 2, hipMemcpyDeviceToHost));
