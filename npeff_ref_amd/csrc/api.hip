@@ -90,6 +90,7 @@ struct dnpeff_nmf {
   float* GH = nullptr;       // [r, r] H^T H from the fused H update (valid while gh_valid)
   float* gpart = nullptr;    // its partial sums
   bool gh_valid = false;
+  bool nw_valid = false;     // Nw holds A H^T of the current H (left there by the loss)
   double sq_norm_A = 0.0;
   Profiler prof;
 };
@@ -163,6 +164,7 @@ DN_API int dnpeff_nmf_init_factors(dnpeff_nmf* nmf) {
   clear_error();
   DN_CHECK(nmf != nullptr, "handle is NULL");
   nmf->gh_valid = false;
+  nmf->nw_valid = false;
   DN_TRY(launch_init_uniform(0, nmf->n, nmf->r, nmf->seed, nmf->W));
   DN_TRY(launch_init_uniform(1, nmf->r, nmf->m, nmf->seed, nmf->H));
   return 0;
@@ -176,6 +178,7 @@ DN_API int dnpeff_nmf_set_factors(dnpeff_nmf* nmf, const float* W_nr, const floa
     DN_HIP(hipMemcpy(nmf->W, W_nr, sizeof(float) * nmf->n * nmf->r, hipMemcpyHostToDevice));
   if (H_rm) {
     nmf->gh_valid = false;
+    nmf->nw_valid = false;
     DN_HIP(hipMemcpy(nmf->S, H_rm, sizeof(float) * nmf->m * nmf->r, hipMemcpyHostToDevice));
     DN_TRY(launch_transpose(nmf->r, nmf->m, nmf->S, nmf->H));
     DN_HIP(hipStreamSynchronize(stream()));
@@ -186,12 +189,15 @@ DN_API int dnpeff_nmf_set_factors(dnpeff_nmf* nmf, const float* W_nr, const floa
 DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
-  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N));
-  DN_TRY(launch_spmm_n(A, h->r, h->H));
-  DN_TRY(h->prof.end());
-  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N_REDUCE));
-  DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
-  DN_TRY(h->prof.end());
+  if (!h->nw_valid) {  // a loss evaluation since the last H update has left A H^T in Nw
+    DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N));
+    DN_TRY(launch_spmm_n(A, h->r, h->H));
+    DN_TRY(h->prof.end());
+    DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N_REDUCE));
+    DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
+    DN_TRY(h->prof.end());
+    h->nw_valid = true;
+  }
   const float* Gh = h->GH;
   if (!h->gh_valid) {
     DN_TRY(h->prof.begin(DNPEFF_K_GRAM_H));
@@ -225,6 +231,7 @@ DN_API int dnpeff_nmf_update_H(dnpeff_nmf* h) {
   }
   DN_TRY(h->prof.end());
   std::swap(h->H, h->S);
+  h->nw_valid = false;
   return 0;
 }
 
@@ -243,8 +250,11 @@ DN_API int dnpeff_nmf_loss_terms(dnpeff_nmf* h, double* sq_norm_A, double* pos, 
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
   // neg = <W^T A, H> = <A H^T, W>
-  DN_TRY(launch_spmm_n(A, h->r, h->H));
-  DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
+  if (!h->nw_valid) {
+    DN_TRY(launch_spmm_n(A, h->r, h->H));
+    DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
+    h->nw_valid = true;
+  }
   DN_TRY(launch_dot(h->n * h->r, h->Nw, h->W, h->dot_ws, h->dot_ws + DOT_BLOCKS));
   // pos = <H, (W^T W) H> = <W^T W, H H^T>
   // (H^T H of the current H is at hand when the last H update produced it)

@@ -99,6 +99,34 @@ def test_run_is_reproducible_bit_for_bit():
     assert outs[0][2] == outs[1][2]
 
 
+@pytest.mark.parametrize("rank", [64, 128])
+def test_loss_evaluations_do_not_change_the_run(rank):
+    """The loss leaves A H^T behind for the next W update (and takes H^T H from the fused H update
+    at rank 128): a run that evaluates the loss after every step and between the two updates ends
+    on the same bits as one that never does, and the loss values agree with a fresh evaluation."""
+    outs = []
+    for with_loss in (False, True):
+        A, norms = d.Csr.synth(200, 150000, k_fixed=1500, seed=9)
+        A.normalize_rows(norms)
+        A.compact_columns(1)
+        nmf = d.MuNmf(A, d.MuNmfParams(rank=rank, max_iters=4, log_every=0))
+        nmf.initialize()
+        losses = []
+        for _ in range(4):
+            nmf.update_W()
+            if with_loss:
+                losses.append(nmf.computeUncachedLoss())
+            nmf.update_H()
+            if with_loss:
+                losses.append(nmf.computeUncachedLoss())
+                losses.append(nmf.computeUncachedLoss())  # twice: everything cached
+        outs.append((nmf.loadWToHostSync(), nmf.loadHToHostSync(), nmf.computeUncachedLoss(), losses))
+        nmf.close()
+        A.close()
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    assert outs[0][2] == outs[1][2] == outs[1][3][-1] == outs[1][3][-2]
+
+
 def test_more_rows_than_columns_is_refused():
     A = d.Csr.from_host([0, 1, 2, 3], [0, 1, 0], [1.0, 1.0, 1.0], 2)
     with pytest.raises(d.DnpeffError, match="more rows than columns"):
