@@ -134,6 +134,19 @@ struct dense_head {
   int64_t ws_floats = 0;
 };
 
+// How the columns of a sparse part are cut into panels for A H^T: `coarse` panels with equal
+// numbers of entries; a coarse panel wider than sweep_cols columns in which a row holds at least
+// sweep_min entries per sweep_cols columns on average is cut into pieces of at most sweep_cols
+// columns, which are swept (spmm.hip).
+struct panel_plan {
+  int coarse = 0;
+  int sweep_cols = 0;
+  double sweep_min = 0.0;
+  bool operator==(const panel_plan& o) const {
+    return coarse == o.coarse && sweep_cols == o.sweep_cols && sweep_min == o.sweep_min;
+  }
+};
+
 }  // namespace dn
 
 struct dnpeff_csr {
@@ -162,6 +175,12 @@ struct dnpeff_csr {
   // inside a panel), seg[row * (n_panels + 1) + p] = first entry of the (row, p) segment
   int n_panels = 0;
   int32_t* panel_bounds = nullptr;  // [n_panels + 1] first column of each panel
+  // panel_ids[0 .. n_plain): panels handled one wave per (row, panel) segment, in grid order;
+  // panel_ids[n_plain .. n_plain + n_swept): swept panels
+  int n_plain = 0, n_swept = 0;
+  int32_t* panel_ids = nullptr;
+  int* sweep_progress = nullptr;  // per-XCD counters of the sweep kernel (256 ints)
+  dn::panel_plan plan;
   int64_t* seg = nullptr;
   int32_t* pcol = nullptr;
   float* pval = nullptr;
@@ -177,8 +196,15 @@ inline const dnpeff_csr* sparse_part(const dnpeff_csr* A) { return A->tail ? A->
 int csr_ensure_chunks(dnpeff_csr* A);
 int csr_ensure_partials(dnpeff_csr* A, int r);
 // Builds (or drops) the column panels of a matrix without dense head / of a sparse part;
-// needs the transposed copy.  n_panels = 0 removes them.
-int csr_set_panels(dnpeff_csr* S, int n_panels);
+// needs the transposed copy.  plan.coarse = 0 removes them.
+int csr_set_panels(dnpeff_csr* S, const panel_plan& plan);
+// Swept panels are summed per XCD: one slot of partial sums per plain panel plus SWEEP_XCDS.
+constexpr int SWEEP_XCDS = 8;
+inline int64_t panel_slots(const dnpeff_csr* S) {
+  return S->n_plain + (S->n_swept > 0 ? SWEEP_XCDS : 0);
+}
+// Ranks the sweep kernel of A H^T handles.
+inline bool spmm_n_sweep_supported(int r) { return r == 32 || r == 64 || r == 128 || r == 256; }
 // Everything A H^T and A^T W at rank r need: transposed copy and work lists of the sparse part,
 // workspaces of the sparse part and of the dense head.
 int csr_ensure_products(dnpeff_csr* A, int r);

@@ -193,7 +193,7 @@ __global__ void __launch_bounds__(256)
 // pass, a scan over the panels, then tiles of 256 entries in order; within a tile an entry's
 // rank among the entries of its panel comes from wave ballots over the bits of the panel
 // number plus the per-wave counts of the earlier waves.
-constexpr int MAX_PANELS = 512;
+constexpr int MAX_PANELS = 3072;
 
 __global__ void __launch_bounds__(256)
     k_panel_split(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
@@ -202,8 +202,8 @@ __global__ void __launch_bounds__(256)
                   int32_t* __restrict__ pcol, float* __restrict__ pval) {
   __shared__ int32_t bnd[MAX_PANELS + 1];
   __shared__ int hist[MAX_PANELS];
-  __shared__ int64_t cursor[MAX_PANELS];
-  __shared__ int wcnt[4][MAX_PANELS];
+  __shared__ int cursor[MAX_PANELS];         // next free position of each panel, relative to e0
+  __shared__ uint8_t wcnt[4][MAX_PANELS];    // entries of a panel in one wave of a tile (<= 64)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   for (int i = tid; i <= P; i += 256) bnd[i] = bounds[i];
   auto panel_of = [&](int32_t col) {
@@ -224,11 +224,32 @@ __global__ void __launch_bounds__(256)
     __syncthreads();
     for (int64_t e = e0 + tid; e < e1; e += 256) atomicAdd(&hist[panel_of(colind[e])], 1);
     __syncthreads();
-    for (int i = tid; i < P; i += 256) {
-      int64_t s = 0;
-      for (int q = 0; q < i; q++) s += hist[q];
-      cursor[i] = e0 + s;
-      seg[row * (P + 1) + i] = e0 + s;
+    // exclusive scan of the panel counts: each thread sums a run of consecutive panels, the
+    // run totals are scanned by thread 0
+    {
+      const int per = (P + 255) / 256, p0 = tid * per;
+      int s = 0;
+      for (int q = p0; q < p0 + per && q < P; q++) s += hist[q];
+      __syncthreads();
+      if (p0 < P) cursor[p0] = s;  // run total, parked in the run's first slot
+      __syncthreads();
+      if (tid == 0) {
+        int run = 0;
+        for (int q = 0; q < P; q += per) {
+          const int t = cursor[q];
+          cursor[q] = run;
+          run += t;
+        }
+      }
+      __syncthreads();
+      if (p0 < P) {
+        int run = cursor[p0];
+        for (int q = p0; q < p0 + per && q < P; q++) {
+          cursor[q] = run;
+          seg[row * (P + 1) + q] = e0 + run;
+          run += hist[q];
+        }
+      }
     }
     if (tid == 0) seg[row * (P + 1) + P] = e1;
     __syncthreads();
@@ -250,24 +271,29 @@ __global__ void __launch_bounds__(256)
         mask &= bit ? bal : ~bal;
       }
       const int rank = __popcll(mask & ((1ull << lane) - 1ull));
-      if (active && rank == 0) wcnt[wave][pid] = __popcll(mask);
+      if (active && rank == 0) wcnt[wave][pid] = (uint8_t)__popcll(mask);
       __syncthreads();
+      int off = 0, tot = 0;
       if (active) {
-        int off = 0;
-        for (int w = 0; w < wave; w++) off += wcnt[w][pid];
-        const int64_t pos = cursor[pid] + off + rank;
+        for (int w = 0; w < 4; w++) {
+          const int c = wcnt[w][pid];
+          if (w < wave) off += c;
+          tot += c;
+        }
+        const int64_t pos = e0 + cursor[pid] + off + rank;
         pcol[pos] = col;
         pval[pos] = v;
       }
       __syncthreads();
-      for (int i = tid; i < P; i += 256) {
-        const int tot = wcnt[0][i] + wcnt[1][i] + wcnt[2][i] + wcnt[3][i];
-        if (tot) {
-          cursor[i] += tot;
-          wcnt[0][i] = wcnt[1][i] = wcnt[2][i] = wcnt[3][i] = 0;
-        }
+      // the last entry of each panel in the tile (last wave that holds it, last lane of its
+      // mask) moves the panel's cursor on and clears its counts
+      if (active) {
+        bool last_wave = true;
+        for (int w = wave + 1; w < 4; w++) last_wave = last_wave && wcnt[w][pid] == 0;
+        if (last_wave && rank == __popcll(mask) - 1) cursor[pid] += tot;
       }
       __syncthreads();
+      if (active && rank == 0) wcnt[wave][pid] = 0;
     }
   }
 }
@@ -430,13 +456,16 @@ static void drop_head(dnpeff_csr* A) {
 
 static void drop_panels(dnpeff_csr* A) {
   dfree(A->panel_bounds); A->panel_bounds = nullptr;
+  dfree(A->panel_ids); A->panel_ids = nullptr;
+  dfree(A->sweep_progress); A->sweep_progress = nullptr;
   dfree(A->seg); A->seg = nullptr;
   dfree(A->pcol); A->pcol = nullptr;
   dfree(A->pval); A->pval = nullptr;
   if (A->n_panels) {  // the partial sums were sized for the panels
     dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
   }
-  A->n_panels = 0;
+  A->n_panels = A->n_plain = A->n_swept = 0;
+  A->plan = panel_plan();
 }
 
 static void drop_derived(dnpeff_csr* A) {
@@ -460,42 +489,96 @@ int csr_ensure_chunks(dnpeff_csr* A) {
   return 0;
 }
 
-int csr_set_panels(dnpeff_csr* S, int P) {
-  if (P == S->n_panels) return 0;
+int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
+  if (plan == S->plan) return 0;
   drop_panels(S);
-  if (P <= 0) return 0;
-  DN_CHECK(P <= MAX_PANELS, "at most %d column panels", MAX_PANELS);
+  const int P0 = plan.coarse;
+  if (P0 <= 0) return 0;
+  DN_CHECK(P0 <= MAX_PANELS, "at most %d column panels", MAX_PANELS);
   DN_CHECK(S->rowptr && S->colptr, "column panels need both copies of the matrix");
   hipStream_t st = stream();
+  // coarse panels: equal numbers of entries
+  std::vector<int32_t> coarse((size_t)P0 + 1);
+  {
+    int32_t* d_coarse = nullptr;
+    DN_TRY(dmalloc(&d_coarse, (int64_t)P0 + 1));
+    hipLaunchKernelGGL(k_panel_bounds, dim3((unsigned)ceil_div(P0 + 1, 256)), dim3(256), 0, st,
+                       S->colptr, S->n_cols, S->nnz, P0, d_coarse);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e == hipSuccess)
+      e = hipMemcpy(coarse.data(), d_coarse, sizeof(int32_t) * coarse.size(), hipMemcpyDeviceToHost);
+    dfree(d_coarse);
+    DN_CHECK(e == hipSuccess, "building the column panels failed: %s", hipGetErrorString(e));
+  }
+  // A coarse panel whose part of the factor does not fit one L2 is cut into pieces that do, when
+  // the rows hold entries enough per piece to be worth a segment each; those pieces are swept
+  // (spmm.hip).  A raised threshold keeps the number of panels within bounds.
+  std::vector<int32_t> bounds, ids, swept;
+  double min_seg = plan.sweep_min;
+  for (;;) {
+    bounds.clear(); ids.clear(); swept.clear();
+    const double per_coarse = (double)S->nnz / P0 / (double)(S->n_rows > 0 ? S->n_rows : 1);
+    for (int c = 0; c < P0; c++) {
+      const int64_t w = (int64_t)coarse[c + 1] - coarse[c];
+      const bool sweep = plan.sweep_cols > 0 && w > plan.sweep_cols + plan.sweep_cols / 4 &&
+                         per_coarse * (double)plan.sweep_cols / (double)w >= min_seg;
+      const int64_t parts = sweep ? ceil_div(w, plan.sweep_cols) : 1;
+      for (int64_t q = 0; q < parts; q++) {
+        (sweep ? swept : ids).push_back((int32_t)bounds.size());
+        bounds.push_back((int32_t)(coarse[c] + w * q / parts));
+      }
+    }
+    if ((int64_t)bounds.size() <= MAX_PANELS) break;
+    min_seg = min_seg > 0.0 ? min_seg * 1.5 : 1.0;
+  }
+  bounds.push_back((int32_t)S->n_cols);
+  const int P = (int)bounds.size() - 1;
+  const int n_plain = (int)ids.size(), n_swept = (int)swept.size();
+  ids.insert(ids.end(), swept.begin(), swept.end());
+
   int bits = 0;
   while ((1 << bits) < P) bits++;
-  int s = dmalloc(&S->panel_bounds, (int64_t)P + 1) || dmalloc(&S->seg, S->n_rows * (P + 1)) ||
-          dmalloc(&S->pcol, S->nnz) || dmalloc(&S->pval, S->nnz);
+  int s = dmalloc(&S->panel_bounds, (int64_t)P + 1) || dmalloc(&S->panel_ids, (int64_t)P) ||
+          dmalloc(&S->sweep_progress, 256) ||
+          dmalloc(&S->seg, S->n_rows * (P + 1)) || dmalloc(&S->pcol, S->nnz + 64) ||
+          dmalloc(&S->pval, S->nnz + 64);  // (the sweep kernel reads 64 pairs at a time)
   if (!s) {
-    hipLaunchKernelGGL(k_panel_bounds, dim3((unsigned)ceil_div(P + 1, 256)), dim3(256), 0, st,
-                       S->colptr, S->n_cols, S->nnz, P, S->panel_bounds);
-    int64_t wgs = S->n_rows < 8192 ? S->n_rows : 8192;
-    hipLaunchKernelGGL(k_panel_split, dim3((unsigned)(wgs < 1 ? 1 : wgs)), dim3(256), 0, st, S->rowptr,
-                       S->colind, S->vals, S->n_rows, P, bits, S->panel_bounds, S->seg, S->pcol,
-                       S->pval);
-    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(st) != hipSuccess) {
-      set_error("building the column panels failed");
+    hipError_t e = hipMemcpy(S->panel_bounds, bounds.data(), sizeof(int32_t) * bounds.size(),
+                             hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+      e = hipMemcpy(S->panel_ids, ids.data(), sizeof(int32_t) * ids.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+      int64_t wgs = S->n_rows < 8192 ? S->n_rows : 8192;
+      hipLaunchKernelGGL(k_panel_split, dim3((unsigned)(wgs < 1 ? 1 : wgs)), dim3(256), 0, st,
+                         S->rowptr, S->colind, S->vals, S->n_rows, P, bits, S->panel_bounds, S->seg,
+                         S->pcol, S->pval);
+      e = hipGetLastError();
+      if (e == hipSuccess) e = hipStreamSynchronize(st);
+    }
+    if (e != hipSuccess) {
+      set_error("building the column panels failed: %s", hipGetErrorString(e));
       s = 1;
     }
   }
   if (s) { drop_panels(S); return s; }
   S->n_panels = P;
+  S->n_plain = n_plain;
+  S->n_swept = n_swept;
+  S->plan = plan;
   dfree(S->partials); S->partials = nullptr; S->partials_floats = 0;
   return 0;
 }
 
 // Panels pay when the gathered factor [n_cols, r] is far larger than the caches and there are
-// rows enough to share a panel's part of it: one panel per ~48 MB of the factor, 8..512, and
-// few enough for the (panel, 4 rows) workgroups to fit one launch.  On 10,000 x 65.9M, r = 128
-// (33.7 GB factor): no panels 29.3 ms, 32: 27.8, 128: 23.9, 256: 21.8, 512: 20.1 ms for the
-// gathers, plus 0.1 to 0.8 ms for the sum over panels; 1024 gains 1.1 ms and loses 0.7.
-// DNPEFF_PANELS overrides the number (0 = none).
-static int panel_policy(const dnpeff_csr* S, int r) {
+// rows enough to share a panel's part of it: one coarse panel per ~48 MB of the factor, 8..512,
+// and few enough for the (panel, 4 rows) workgroups to fit one launch.  On 10,000 x 65.9M,
+// r = 128 (33.7 GB factor): no panels 29.3 ms, 32: 27.8, 128: 23.9, 256: 21.8, 512: 20.1 ms for
+// the gathers, plus 0.1 to 0.8 ms for the sum over panels; 1024 gains 1.1 ms and loses 0.7.
+// DNPEFF_PANELS overrides the number (0 = none).  Swept pieces hold DNPEFF_SWEEP_BYTES of the
+// factor each (default 3 MB of the 4 MB L2 of an XCD; 0 = no sweeps) and are made where a row
+// holds DNPEFF_SWEEP_MIN entries per piece on average.
+static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   int64_t P = 0;
   const double bytes = 4.0 * (double)S->n_cols * r;
   if (bytes >= 512e6 && S->n_rows >= 64) {
@@ -503,11 +586,22 @@ static int panel_policy(const dnpeff_csr* S, int r) {
     if (P < 8) P = 8;
   }
   if (const char* e = getenv("DNPEFF_PANELS")) P = atoi(e);
-  if (P > MAX_PANELS) P = MAX_PANELS;
+  if (P > 512) P = 512;
   const int64_t row_groups = ceil_div(S->n_rows, 4);
   while (P > 1 && P * row_groups >= ((int64_t)1 << 24)) P /= 2;
   if (P < 2 || S->nnz == 0) P = 0;
-  return (int)P;
+  panel_plan plan;
+  plan.coarse = (int)P;
+  if (P > 0 && spmm_n_sweep_supported(r)) {
+    double sweep_bytes = 3.0 * 1024 * 1024;
+    if (const char* e = getenv("DNPEFF_SWEEP_BYTES")) sweep_bytes = atof(e);
+    if (sweep_bytes > 1e9) sweep_bytes = 1e9;  // (the kernel addresses a piece with 32 bits)
+    plan.sweep_cols = (int)(sweep_bytes / (4.0 * r));
+    plan.sweep_min = 4.0;
+    if (const char* e = getenv("DNPEFF_SWEEP_MIN")) plan.sweep_min = atof(e);
+    if (plan.sweep_cols <= 0) plan.sweep_cols = 0, plan.sweep_min = 0.0;
+  }
+  return plan;
 }
 
 int csr_ensure_products(dnpeff_csr* A, int r) {
@@ -521,8 +615,8 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
 int csr_ensure_partials(dnpeff_csr* A, int r) {
   DN_TRY(csr_ensure_chunks(A));
   int64_t need = A->n_chunks * (int64_t)r;
-  if (A->n_panels > 0 && A->n_rows * A->n_panels * (int64_t)r > need)
-    need = A->n_rows * A->n_panels * (int64_t)r;
+  if (A->n_panels > 0 && A->n_rows * panel_slots(A) * (int64_t)r > need)
+    need = A->n_rows * panel_slots(A) * (int64_t)r;
   if (need <= A->partials_floats && A->partials) return 0;
   dfree(A->partials);
   A->partials = nullptr;

@@ -11,6 +11,7 @@
 #include "dnpeff_internal.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace dn {
 
@@ -235,17 +236,263 @@ __global__ void __launch_bounds__(256)
 template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_n_panel(const int64_t* __restrict__ seg, const int32_t* __restrict__ pcol,
-                   const float* __restrict__ pval, int64_t n_rows, int64_t row_groups, int P, int r,
-                   const float* __restrict__ H, float* __restrict__ part) {
+                   const float* __restrict__ pval, int64_t n_rows, int64_t row_groups, int P,
+                   const int32_t* __restrict__ ids, int slots, int r, const float* __restrict__ H,
+                   float* __restrict__ part) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int64_t p = blockIdx.x / row_groups;
+  const int64_t slot = blockIdx.x / row_groups;
   const int64_t row = (blockIdx.x % row_groups) * 4 + wave;
   if (row >= n_rows) return;
-  const int64_t* sg = seg + row * (P + 1) + p;
+  const int64_t* sg = seg + row * (P + 1) + ids[slot];
   GT g;
   g.init(lane, r);
   g.run(pcol, pval, sg[0], sg[1], H, r);
-  g.store(part + (row * P + p) * r);
+  g.store(part + (row * slots + slot) * r);
+}
+
+// ---------------------------------------------------------------------------
+// Swept panels.  Where a coarse panel's part of H is larger than an L2 and its columns still
+// hold several entries each, the panel is cut into pieces that fit the 4 MB L2 of one XCD, and
+// XCD x (workgroups x, x + 8, ... : the dispatcher deals workgroups to the XCDs round-robin)
+// takes pieces x, x + 8, ... one after the other, for all rows of a pass: the rows of H of a
+// piece then come from that XCD's L2 for every row after the first that uses them.
+//
+// All workgroups of the grid are resident at once (two per CU) and a workgroup keeps the running
+// sums of its rows in LDS for the whole sweep, so nothing is written until the end of the pass.
+// A wave owns the rows i * waves + wave of its workgroup and handles their (row, piece) segments
+// one after the other: LPR = r / 4 lanes gather one row of H with 16-byte loads, the 64 / LPR
+// lane groups take the entries of the segment round-robin and are added in a fixed butterfly
+// order before the segment's sum goes to LDS.  The (column, value) pairs of a segment are
+// requested two segments ahead and the segment offsets of a piece two pieces ahead, both right
+// after a batch of gathers has been issued: loads return in order, so a request from HBM placed
+// before gathers would hold those up.
+//
+// The workgroups of an XCD keep within `lag` pieces of each other: workgroups that ran ahead
+// (their rows hold fewer entries) would otherwise widen the part of H in use beyond the L2.
+// Each workgroup counts its finished pieces into a per-XCD counter and starts piece i only when
+// the count says that all have finished piece i - 1 - lag.  The counter is only used by
+// workgroups of one XCD, which share an L2, so it is bumped and polled with L2 atomics of
+// workgroup scope (device scope costs a trip to the memory side per poll).  The wait is bounded
+// (spin_max polls): a grid that is not resident as a whole is slow but ends, and the sums do not
+// depend on the counter.  One partial sum per (row, XCD): part[row, slot0 + x, :].
+// ---------------------------------------------------------------------------
+constexpr int SWEEP_SYNC_STRIDE = 32;    // ints between the progress counters of two XCDs
+constexpr int SWEEP_LDS_BYTES = 81920;   // running sums of a workgroup: half the LDS of a CU
+constexpr int SWEEP_MAX_SEGS = 32;       // rows per wave (their offsets live in the 64 lanes)
+
+template <int LPR, bool A16>
+__global__ void __launch_bounds__(1024)
+    k_spmm_n_sweep(const int64_t* __restrict__ seg, const int32_t* __restrict__ pcol,
+                   const float* __restrict__ pval, int64_t row0, int64_t row1, int P,
+                   const int32_t* __restrict__ swept, int n_swept,
+                   const int32_t* __restrict__ bounds_of, int slots, int slot0, int r,
+                   const float* __restrict__ H, float* __restrict__ part,
+                   int* __restrict__ progress, int lag, int spin_max, int rows_wg) {
+  extern __shared__ __align__(16) float sums[];  // [rows_wg][r], row l = i * waves + wave
+  constexpr int G = 64 / LPR;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int waves = blockDim.x >> 6;
+  const int sub = lane % LPR, grp = lane / LPR;
+  const int x = blockIdx.x % SWEEP_XCDS;
+  const int64_t q = blockIdx.x / SWEEP_XCDS, nq = gridDim.x / SWEEP_XCDS;
+  int* const counter = progress + x * SWEEP_SYNC_STRIDE;
+  const int n_pi = (n_swept - x + SWEEP_XCDS - 1) / SWEEP_XCDS;  // pieces of this XCD
+  auto row_of = [&](int i) { return row0 + ((int64_t)i * waves + wave) * nq + q; };
+  // rows of this wave: those with i * waves + wave < rows_wg (at least two, at most 32)
+  const int n_i = (rows_wg - wave + waves - 1) / waves;
+
+  for (int i = 0; i < n_i; i++)
+    for (int c = lane; c < r; c += 64) sums[(size_t)(i * waves + wave) * r + c] = 0.0f;
+
+  // Segment bounds live in the lanes: lane i holds the first pair and the length of the
+  // (row_i, piece) segment of the current piece, lane 32 + i those of the next piece; a third
+  // set (in the upper lanes of `st_*`) is on its way for the piece after that.  Lanes without a
+  // row and pieces past the end hold empty segments.
+  const int64_t my_row = row_of(lane & 31);
+  const bool my_seg = (lane & 31) < n_i && my_row < row1;
+  auto load_off = [&](int pi, int64_t& s0, int& len) {
+    const bool ok = my_seg && pi < n_pi;
+    const int piece = swept[x + SWEEP_XCDS * (pi < n_pi ? pi : 0)];
+    const int64_t at = ok ? my_row * (P + 1) + piece : 0;
+    const int64_t a = seg[at], b = seg[at + 1];
+    s0 = ok ? a : 0;
+    len = ok ? (int)(b - a) : 0;
+  };
+  auto bcast_i64 = [&](int64_t v, int src) {
+    const int lo = (int)(uint32_t)(v & 0xffffffffLL), hi = (int)(v >> 32);
+    return ((int64_t)bcast_i(hi, src) << 32) | (uint32_t)bcast_i(lo, src);
+  };
+  const unsigned r4 = 4u * (unsigned)r, sub16 = 16u * (unsigned)sub;
+
+  if (n_pi > 0) {  // (n_pi is the same for all waves of the workgroup)
+    int64_t cm_s0, st_s0;
+    int cm_len, st_len;
+    {
+      int64_t s0a, s0b;
+      int lena, lenb;
+      load_off(0, s0a, lena);
+      load_off(1, s0b, lenb);
+      cm_s0 = lane < 32 ? s0a : s0b;
+      cm_len = lane < 32 ? lena : lenb;
+      load_off(2, st_s0, st_len);
+    }
+    int pi = 0, i = 0;
+    // rows of H of the current piece: Hp + 4 r (column - c0), a 32-bit offset
+    int c0 = bounds_of[swept[x]];
+    const char* Hp = reinterpret_cast<const char*>(H + (int64_t)c0 * r);
+    int ra_i, rb_i;
+    float ra_v, rb_v;
+    ra_i = (pcol + bcast_i64(cm_s0, 0))[lane];
+    ra_v = (pval + bcast_i64(cm_s0, 0))[lane];
+    rb_i = (pcol + bcast_i64(cm_s0, 1))[lane];  // (a wave owns at least two rows)
+    rb_v = (pval + bcast_i64(cm_s0, 1))[lane];
+    // One segment: (ri, rv) hold its first 64 pairs (and whatever follows them in memory: the
+    // arrays end with 64 spare pairs) and are refilled with those of the segment after the next.
+    auto segment = [&](int& ri, float& rv) {
+      if (i == 0 && pi > lag) {
+        if (threadIdx.x == 0) {
+          const int want = (int)nq * (pi - lag);
+          for (int spin = 0; spin < spin_max; spin++) {
+            // an L2 atomic that changes nothing (the counter is never negative) reads the counter
+            if (__hip_atomic_fetch_max(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >=
+                want)
+              break;
+            __builtin_amdgcn_s_sleep(8);
+          }
+        }
+        __syncthreads();
+      }
+      const int64_t s0 = bcast_i64(cm_s0, i);
+      const int len = bcast_i(cm_len, i);
+      // the segment after the next: two rows on, possibly in the next piece
+      const int l2 = i + 2 < n_i ? i + 2 : 32 + i + 2 - n_i;
+      const int32_t* pc2 = pcol + bcast_i64(cm_s0, l2);
+      const float* pv2 = pval + bcast_i64(cm_s0, l2);
+
+      float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      // lanes past the segment hold (first row of the piece, value 0): a padded step gathers
+      // that row with weight 0
+      int my_i = lane < len ? ri - c0 : 0;
+      float my_v = lane < len ? rv : 0.0f;
+      auto gathers = [&](auto u_tag, int st, float4* h, float* a) {
+        constexpr int U = decltype(u_tag)::value;
+#pragma unroll
+        for (int uu = 0; uu < U; uu++) {
+          const int u = ((st + uu) * G + grp) & 63;
+          a[uu] = __shfl(my_v, u);
+          const unsigned at = __umul24((unsigned)__shfl(my_i, u), r4) + sub16;
+          const float* hx = reinterpret_cast<const float*>(Hp + at);
+          if (A16) {
+            h[uu] = *reinterpret_cast<const float4*>(hx);
+          } else {
+            h[uu] = make_float4(hx[0], hx[1], hx[2], hx[3]);
+          }
+        }
+      };
+      auto sums_up = [&](auto u_tag, const float4* h, const float* a) {
+        constexpr int U = decltype(u_tag)::value;
+#pragma unroll
+        for (int uu = 0; uu < U; uu++) {
+          acc.x = fmaf(a[uu], h[uu].x, acc.x);
+          acc.y = fmaf(a[uu], h[uu].y, acc.y);
+          acc.z = fmaf(a[uu], h[uu].z, acc.z);
+          acc.w = fmaf(a[uu], h[uu].w, acc.w);
+        }
+      };
+      using U2 = std::integral_constant<int, 2>;
+      using U4 = std::integral_constant<int, 4>;
+      // the first gathers of the segment and their sums, then the request for the segment
+      // after the next
+      int nsteps = ((len < 64 ? len : 64) + G - 1) / G;
+      int st;
+      if (nsteps > 2) {
+        float4 h[4];
+        float a[4];
+        gathers(U4{}, 0, h, a);
+        sums_up(U4{}, h, a);
+        st = 4;
+      } else {
+        float4 h[2];
+        float a[2];
+        gathers(U2{}, 0, h, a);
+        sums_up(U2{}, h, a);
+        st = 2;
+      }
+      ri = pc2[lane];
+      rv = pv2[lane];
+      for (int base = 0; base < len; base += 64) {
+        if (base > 0) {
+          my_i = (pcol + s0)[base + lane];
+          my_v = (pval + s0)[base + lane];
+          my_i = base + lane < len ? my_i - c0 : 0;
+          my_v = base + lane < len ? my_v : 0.0f;
+          nsteps = ((len - base < 64 ? len - base : 64) + G - 1) / G;
+          st = 0;
+        }
+        while (st < nsteps) {
+          if (nsteps - st > 2) {
+            float4 h[4];
+            float a[4];
+            gathers(U4{}, st, h, a);
+            sums_up(U4{}, h, a);
+            st += 4;
+          } else {
+            float4 h[2];
+            float a[2];
+            gathers(U2{}, st, h, a);
+            sums_up(U2{}, h, a);
+            st += 2;
+          }
+        }
+      }
+      if (len > 0) {
+#pragma unroll
+        for (int off = 32; off >= LPR; off >>= 1) {
+          acc.x += __shfl_xor(acc.x, off);
+          acc.y += __shfl_xor(acc.y, off);
+          acc.z += __shfl_xor(acc.z, off);
+          acc.w += __shfl_xor(acc.w, off);
+        }
+        if (grp == 0) {
+          float4* dst = reinterpret_cast<float4*>(sums + (size_t)(i * waves + wave) * r) + sub;
+          float4 t = *dst;
+          t.x += acc.x; t.y += acc.y; t.z += acc.z; t.w += acc.w;
+          *dst = t;
+        }
+      }
+      if (++i == n_i) {  // the piece is done
+        // bounds: the next piece moves to the lower lanes, the one after it to the upper lanes,
+        // and the request for a further one goes out before the wait for the other workgroups
+        const int64_t lo_s0 = (int64_t)(((uint64_t)(uint32_t)__shfl((int)(cm_s0 >> 32), lane + 32) << 32) |
+                                        (uint32_t)__shfl((int)(uint32_t)(cm_s0 & 0xffffffffLL), lane + 32));
+        const int lo_len = __shfl(cm_len, lane + 32);
+        cm_s0 = lane < 32 ? lo_s0 : st_s0;
+        cm_len = lane < 32 ? lo_len : st_len;
+        i = 0;
+        pi++;
+        load_off(pi + 2, st_s0, st_len);
+        c0 = bounds_of[swept[x + SWEEP_XCDS * (pi < n_pi ? pi : 0)]];
+        Hp = reinterpret_cast<const char*>(H + (int64_t)c0 * r);
+        __syncthreads();
+        if (threadIdx.x == 0)
+          __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    };
+    const int total = n_pi * n_i;
+    for (int t = 0; t < total; t += 2) {
+      segment(ra_i, ra_v);
+      if (t + 1 < total) segment(rb_i, rb_v);
+    }
+  }
+
+  for (int i = 0; i < n_i; i++) {
+    const int64_t row = row_of(i);
+    if (row < row1) {
+      const float* src = sums + (size_t)(i * waves + wave) * r;
+      float* dst = part + (row * slots + slot0 + x) * r;
+      for (int c = lane; c < r; c += 64) dst[c] = src[c];
+    }
+  }
 }
 
 // N[row, :] = sum of the row's panel partials, in panel order, accumulated in fp64.
@@ -605,22 +852,118 @@ static int dispatch_gather(int r, bool aligned16, F&& f) {
   }
 }
 
+__global__ void k_sweep_clear(int* progress) { progress[threadIdx.x] = 0; }
+
+// Shape of a sweep launch: two workgroups per CU, each with SWEEP_LDS_BYTES of running sums; the
+// number of waves per workgroup is the largest (at most max_waves) that covers the rows in the
+// fewest passes; DNPEFF_SWEEP_WAVES overrides it.  More rows than one launch covers take several
+// passes of equal size.
+struct sweep_shape {
+  int waves, rows_wg;
+  int64_t wgs, n_pass, rows_per_pass;
+};
+// max_waves: the most waves per workgroup that leave two workgroups resident per CU
+static sweep_shape sweep_shape_for(int64_t n_rows, int r, int max_waves) {
+  sweep_shape best{};
+  const int64_t wgs = (int64_t)n_cus() * 2 / SWEEP_XCDS * SWEEP_XCDS;
+  const int rows_cap = SWEEP_LDS_BYTES / (4 * r);
+  int forced = 0;
+  if (const char* e = getenv("DNPEFF_SWEEP_WAVES")) forced = atoi(e);
+  if (forced < 1 || forced > max_waves) forced = 0;
+  for (int waves = max_waves; waves >= 2; waves -= 2) {
+    const int w = forced ? forced : waves;
+    // every wave owns 2 to SWEEP_MAX_SEGS rows: the kernel looks two segments ahead within two
+    // pieces and keeps the segment bounds of a piece in 32 lanes
+    const int rows_wg = rows_cap < SWEEP_MAX_SEGS * w ? rows_cap : SWEEP_MAX_SEGS * w;
+    if (rows_wg >= 2 * w) {
+      const int64_t cover = wgs / SWEEP_XCDS * rows_wg;
+      const int64_t n_pass = ceil_div(n_rows, cover);
+      if (best.waves == 0 || n_pass < best.n_pass) best = sweep_shape{w, rows_wg, wgs, n_pass, 0};
+    }
+    if (forced) break;
+  }
+  best.rows_per_pass = ceil_div(n_rows, best.n_pass > 0 ? best.n_pass : 1);
+  return best;
+}
+
+// Registers per SIMD lane that resident waves can share.  The file holds 512, but a launch of
+// 8 waves per SIMD at 64 registers ran with 7 resident and one of 5 at 96 with 4 (the sweep's
+// workgroups then wait for workgroups that have not started), so the shape is planned for 448.
+constexpr int SWEEP_REGISTER_BUDGET = 448;
+
+using sweep_kernel_t = void (*)(const int64_t*, const int32_t*, const float*, int64_t, int64_t, int,
+                                const int32_t*, int, const int32_t*, int, int, int, const float*,
+                                float*, int*, int, int, int);
+
+static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bool aligned,
+                               int slots) {
+  DN_CHECK(spmm_n_sweep_supported(r), "swept panels at rank %d", r);
+  DN_CHECK(A->sweep_progress != nullptr, "matrix has no sweep counters");
+  sweep_kernel_t kernel = nullptr;
+  switch (r / 4 * 2 + (aligned ? 1 : 0)) {
+    case 8 * 2 + 1: kernel = k_spmm_n_sweep<8, true>; break;
+    case 8 * 2: kernel = k_spmm_n_sweep<8, false>; break;
+    case 16 * 2 + 1: kernel = k_spmm_n_sweep<16, true>; break;
+    case 16 * 2: kernel = k_spmm_n_sweep<16, false>; break;
+    case 32 * 2 + 1: kernel = k_spmm_n_sweep<32, true>; break;
+    case 32 * 2: kernel = k_spmm_n_sweep<32, false>; break;
+    case 64 * 2 + 1: kernel = k_spmm_n_sweep<64, true>; break;
+    default: kernel = k_spmm_n_sweep<64, false>; break;
+  }
+  hipFuncAttributes attr;
+  DN_HIP(hipFuncGetAttributes(&attr, (const void*)kernel));
+  const int regs = (attr.numRegs + 7) / 8 * 8;
+  // two workgroups per CU: a workgroup puts waves / 4 waves on each of the 4 SIMDs
+  int max_waves = SWEEP_REGISTER_BUDGET / (regs > 0 ? regs : 8) * 4 / 2;
+  if (max_waves > 14) max_waves = 14;
+  max_waves &= ~1;
+  DN_CHECK(max_waves >= 2, "the sweep kernel needs %d registers", attr.numRegs);
+  const sweep_shape sh = sweep_shape_for(A->n_rows, r, max_waves);
+  DN_CHECK(sh.waves > 0, "no sweep shape for rank %d", r);
+  const int32_t* swept = A->panel_ids + A->n_plain;
+  int lag = 0, spin_max = 400;
+  if (const char* e = getenv("DNPEFF_SWEEP_LAG")) lag = atoi(e);
+  if (const char* e = getenv("DNPEFF_SWEEP_SPIN")) spin_max = atoi(e);
+  if (lag < 0) lag = 0;
+  const size_t lds = sizeof(float) * (size_t)sh.rows_wg * r;
+  DN_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                             SWEEP_LDS_BYTES));
+  for (int64_t pass = 0; pass < sh.n_pass; pass++) {
+    const int64_t row0 = pass * sh.rows_per_pass;
+    const int64_t row1 = row0 + sh.rows_per_pass < A->n_rows ? row0 + sh.rows_per_pass : A->n_rows;
+    hipLaunchKernelGGL(k_sweep_clear, dim3(1), dim3(SWEEP_XCDS * SWEEP_SYNC_STRIDE), 0, stream(),
+                       A->sweep_progress);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)sh.wgs), dim3(64 * sh.waves), lds, stream(), A->seg,
+                       A->pcol, A->pval, row0, row1, A->n_panels, swept, A->n_swept,
+                       A->panel_bounds, slots, A->n_plain, r, H_mr, A->partials, A->sweep_progress,
+                       lag, spin_max, sh.rows_wg);
+    DN_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
 int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   DN_TRY(launch_head_n(A_full, r, H_mr));
   const dnpeff_csr* A = sparse_part(A_full);
   float* partials = A->partials;
   if (A->n_panels > 0) {
-    DN_CHECK(A->seg && A->pcol && partials, "matrix has no panel work list");
-    const int64_t row_groups = ceil_div(A->n_rows, 4);
-    dim3 grid((unsigned)(row_groups * A->n_panels)), block(256);
-    dispatch_gather(r, ((uintptr_t)H_mr % 16) == 0, [&](auto tag) {
-      using GT = typename decltype(tag)::type;
-      hipLaunchKernelGGL((k_spmm_n_panel<GT>), grid, block, 0, stream(), A->seg, A->pcol, A->pval,
-                         A->n_rows, row_groups, A->n_panels, r, H_mr, partials);
-      return 0;
-    });
-    DN_LAUNCH_CHECK();
+    DN_CHECK(A->seg && A->pcol && A->panel_ids && partials, "matrix has no panel work list");
+    const bool aligned = ((uintptr_t)H_mr % 16) == 0;
+    const int slots = (int)panel_slots(A);
+    if (A->n_plain > 0) {
+      const int64_t row_groups = ceil_div(A->n_rows, 4);
+      dim3 grid((unsigned)(row_groups * A->n_plain)), block(256);
+      dispatch_gather(r, aligned, [&](auto tag) {
+        using GT = typename decltype(tag)::type;
+        hipLaunchKernelGGL((k_spmm_n_panel<GT>), grid, block, 0, stream(), A->seg, A->pcol,
+                           A->pval, A->n_rows, row_groups, A->n_panels, A->panel_ids, slots, r, H_mr,
+                           partials);
+        return 0;
+      });
+      DN_LAUNCH_CHECK();
+    }
+    if (A->n_swept > 0) DN_TRY(launch_spmm_n_sweep(A, r, H_mr, aligned, slots));
     return 0;
   }
   DN_CHECK(A->rowptr && A->chunk_base && partials, "matrix has no row-major copy / work list");
@@ -645,7 +988,7 @@ int launch_spmm_n_reduce(const dnpeff_csr* A_full, int r, float* N_nr) {
       int64_t wgs = ceil_div(A->n_rows * r, 256);
       if (wgs > (1 << 20)) wgs = 1 << 20;
       hipLaunchKernelGGL(k_panel_reduce, dim3((unsigned)wgs), dim3(256), 0, stream(), A->partials,
-                         A->n_rows, A->n_panels, r, N_nr);
+                         A->n_rows, (int)panel_slots(A), r, N_nr);
       DN_LAUNCH_CHECK();
     }
   } else {

@@ -311,6 +311,47 @@ def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
     A.close()
 
 
+@pytest.mark.parametrize("r,n,m,maxk,panels,sweep_bytes,waves", [
+    (128, 2700, 6000, 900, 4, 64 * 512, 1),      # two passes, 64-column pieces
+    (128, 130, 3000, 2500, 3, 300 * 512, 8),     # the 5 segments of a wave hold several batches of 64
+    (64, 1500, 9000, 60, 8, 500 * 256, 1),       # short segments, many empty; 3 lane groups idle
+    (32, 333, 5000, 300, 5, 200 * 128, 2),
+    (256, 90, 2000, 700, 2, 400 * 1024, 8),      # 6 pieces: two XCDs have none
+    (128, 40, 50000, 300, 16, 1000 * 512, 8),
+])
+def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, monkeypatch):
+    """Coarse panels cut into L2-sized pieces that one XCD sweeps for all rows, running sums in
+    registers: same sums as the fp64 restatement, same bits on every run, empty rows included; a
+    factor that is not 16-byte aligned takes the 4-byte loads."""
+    monkeypatch.setenv("DNPEFF_PANELS", str(panels))
+    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", str(sweep_bytes))
+    monkeypatch.setenv("DNPEFF_SWEEP_MIN", "0")
+    monkeypatch.setenv("DNPEFF_SWEEP_WAVES", str(waves))
+    rng = np.random.default_rng(r + n)
+    rp, ci, va = random_csr(rng, n, m, maxk, empty_rows={0, n // 2})
+    A = d.Csr.from_host(rp, ci, va, m)
+    H = rng.random((m, r)).astype(np.float32)
+    dH, dN = d.DeviceArray.from_numpy(H), d.DeviceArray((n, r))
+    d.op_spmm_n(A, r, dH, dN)
+    N = dN.numpy()
+    N64 = orc.spmm_n_f64(rp, ci, va, H)
+    assert (np.abs(N - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
+    assert np.all(N[0] == 0) and np.all(N[n // 2] == 0)
+    d.op_spmm_n(A, r, dH, dN)
+    assert np.array_equal(dN.numpy(), N)
+    # the same factor one float further on: not 16-byte aligned
+    import ctypes, types
+    shifted = d.DeviceArray.from_numpy(np.concatenate([np.zeros(1, np.float32), H.ravel()]))
+    view = types.SimpleNamespace(ptr=ctypes.c_void_p(shifted.ptr.value + 4))
+    d.op_spmm_n(A, r, view, dN)
+    assert (np.abs(dN.numpy() - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
+    # without sweeps: every panel one wave per (row, panel) segment
+    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", "0")
+    d.op_spmm_n(A, r, dH, dN)
+    assert _rel(dN.numpy(), N64) < TOL
+    A.close()
+
+
 def test_column_panels_with_dense_head(monkeypatch):
     monkeypatch.setenv("DNPEFF_PANELS", "16")
     rng = np.random.default_rng(11)
