@@ -577,7 +577,7 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
 // the gathers, plus 0.1 to 0.8 ms for the sum over panels; 1024 gains 1.1 ms and loses 0.7.
 // DNPEFF_PANELS overrides the number (0 = none).  Swept pieces hold DNPEFF_SWEEP_BYTES of the
 // factor each (default 3 MB of the 4 MB L2 of an XCD; 0 = no sweeps) and are made where a row
-// holds DNPEFF_SWEEP_MIN entries per piece on average.
+// holds DNPEFF_SWEEP_MIN entries per piece on average (default 4, more when there are few rows).
 static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   int64_t P = 0;
   const double bytes = 4.0 * (double)S->n_cols * r;
@@ -597,7 +597,11 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
     if (const char* e = getenv("DNPEFF_SWEEP_BYTES")) sweep_bytes = atof(e);
     if (sweep_bytes > 1e9) sweep_bytes = 1e9;  // (the kernel addresses a piece with 32 bits)
     plan.sweep_cols = (int)(sweep_bytes / (4.0 * r));
+    // a piece must also bring work enough for a sweep step (a wait for the other workgroups of
+    // the XCD and two barriers): 20,000 entries over all rows
     plan.sweep_min = 4.0;
+    if (S->n_rows > 0 && 20000.0 / (double)S->n_rows > plan.sweep_min)
+      plan.sweep_min = 20000.0 / (double)S->n_rows;
     if (const char* e = getenv("DNPEFF_SWEEP_MIN")) plan.sweep_min = atof(e);
     if (plan.sweep_cols <= 0) plan.sweep_cols = 0, plan.sweep_min = 0.0;
   }
