@@ -210,6 +210,26 @@ def test_column_panel_run_matches_oracle(monkeypatch):
     A.close()
 
 
+@pytest.mark.parametrize("r,waves", [(128, 14), (64, 3)])
+def test_swept_piece_run_matches_oracle(r, waves, monkeypatch):
+    """Column panels cut into small pieces that the XCDs sweep (forced on: 40 columns per piece,
+    any density): 50 iterations stay within the bar, and a second run gives the same bits."""
+    monkeypatch.setenv("DNPEFF_PANELS", "6")
+    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", str(40 * 4 * r))
+    monkeypatch.setenv("DNPEFF_SWEEP_MIN", "0")
+    monkeypatch.setenv("DNPEFF_SWEEP_WAVES", str(waves))
+    nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(300, 40000, 2048, r, 1e-8, 50, seed=9)
+    assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
+    got = np.array([h[1] for h in hist])
+    assert np.all(np.abs(got - losses64) / losses64 < REL)
+    nmf.close()
+    A.close()
+    nmf2, A2, _, (W2, H2), _, _, _ = _run_case(300, 40000, 2048, r, 1e-8, 50, seed=9)
+    assert np.array_equal(W2, W) and np.array_equal(H2, H)
+    nmf2.close()
+    A2.close()
+
+
 def test_ragged_rows_rank_512(monkeypatch):
     """Row lengths drawn log-uniformly over two decades (the ragged-row case), r = 512: the tiled
     X G kernel, the tile-pair Gram and the grouped A^T W at their widest, with column panels
