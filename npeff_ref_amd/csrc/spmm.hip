@@ -92,8 +92,9 @@ struct GatherDword {
 // loads per lane when the row is wider than 64 such pieces); the wave's 64/LPR
 // lane groups take the entries of a batch round-robin, so group g applies
 // entries g, g + G, g + 2G, ... in order, and the groups are added at the end in
-// a fixed butterfly order.
-template <int LPR, int T>
+// a fixed butterfly order.  FULL: the width is 4 LPR T, every lane holds components and the
+// loads need no predicates.
+template <int LPR, int T, bool FULL = false>
 struct GatherVec4 {
   static constexpr int G = 64 / LPR;
   static constexpr int UNR = T >= 4 ? 1 : T == 2 ? 2 : 4;
@@ -109,7 +110,7 @@ struct GatherVec4 {
     grp = lane / LPR;
 #pragma unroll
     for (int t = 0; t < T; t++) {
-      ok[t] = 4 * (sub + 64 * t) < width;
+      ok[t] = FULL || 4 * (sub + 64 * t) < width;
       acc[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
   }
@@ -140,8 +141,8 @@ struct GatherVec4 {
                                  : X + (int64_t)j * r + 4 * sub;
 #pragma unroll
           for (int t = 0; t < T; t++)
-            h[uu][t] = ok[t] ? *reinterpret_cast<const float4*>(x + 256 * t)
-                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            h[uu][t] = FULL || ok[t] ? *reinterpret_cast<const float4*>(x + 256 * t)
+                                     : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int uu = 0; uu < UNR; uu++)
@@ -170,7 +171,7 @@ struct GatherVec4 {
     if (grp == 0) {
 #pragma unroll
       for (int t = 0; t < T; t++)
-        if (ok[t]) *reinterpret_cast<float4*>(dst + 4 * (sub + 64 * t)) = acc[t];
+        if (FULL || ok[t]) *reinterpret_cast<float4*>(dst + 4 * (sub + 64 * t)) = acc[t];
     }
   }
 };
@@ -561,11 +562,14 @@ __global__ void __launch_bounds__(256)
 // group and gathers each W row with one 16-byte load per lane; entries are applied in order.
 constexpr int SPMM_T_COLS = 32;
 
-template <int LPR, int T>
+// FULL: r = 4 LPR T, every lane holds components (no predicates); SMALL: W has fewer than 2^24
+// rows and 4 GB, a row is addressed as the (uniform) base of W plus a 32-bit offset made by one
+// 24-bit multiply-add.
+template <int LPR, int T, bool FULL, bool SMALL>
 __global__ void __launch_bounds__(256)
     k_spmm_t_grouped(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
                      const float* __restrict__ tvals, int64_t m, int r,
-                     const float* __restrict__ W, float* __restrict__ Tout, bool w_small) {
+                     const float* __restrict__ W, float* __restrict__ Tout) {
   constexpr int G = 64 / LPR;
   constexpr int UNR = T >= 4 ? 1 : T == 2 ? 2 : 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -574,7 +578,8 @@ __global__ void __launch_bounds__(256)
   if (j0 >= m) return;
   bool ok[T];
 #pragma unroll
-  for (int t = 0; t < T; t++) ok[t] = 4 * (sub + LPR * t) < r;
+  for (int t = 0; t < T; t++) ok[t] = FULL || 4 * (sub + LPR * t) < r;
+  const unsigned r4 = 4u * (unsigned)r, sub16 = 16u * (unsigned)sub;
 
   // colptr[j0 + lane] for lane <= SPMM_T_COLS, as two 32-bit halves for the shuffles
   const int64_t jc = j0 + lane < m ? j0 + lane : m;
@@ -639,10 +644,12 @@ __global__ void __launch_bounds__(256)
       // Whole blocks of UNR entries with their loads in flight together, then the rest one by
       // one: most columns hold one or two entries.  Lanes past a group's entries hold
       // (row 0, value 0), so a step that a shorter group only accompanies gathers row 0 with
-      // weight 0 and needs no predicate; offsets into W are 32-bit when W is below 4 GB.
+      // weight 0 and needs no predicate.
       auto wrow = [&](int jrow) {
-        return w_small ? W + ((unsigned)jrow * (unsigned)r + 4u * (unsigned)sub)
-                       : W + (int64_t)jrow * r + 4 * sub;
+        if (SMALL)
+          return reinterpret_cast<const float*>(reinterpret_cast<const char*>(W) +
+                                                (__umul24((unsigned)jrow, r4) + sub16));
+        return W + (int64_t)jrow * r + 4 * sub;
       };
       int u = 0;
       for (; u + UNR <= cmax; u += UNR) {
@@ -654,8 +661,8 @@ __global__ void __launch_bounds__(256)
           a[uu] = __shfl(my_v, gbase + u + uu);
 #pragma unroll
           for (int t = 0; t < T; t++)
-            h[uu][t] = ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
-                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            h[uu][t] = FULL || ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
+                                     : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int uu = 0; uu < UNR; uu++)
@@ -672,8 +679,8 @@ __global__ void __launch_bounds__(256)
         const float a = __shfl(my_v, gbase + u);
 #pragma unroll
         for (int t = 0; t < T; t++) {
-          const float4 h = ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
-                                 : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          const float4 h = FULL || ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
+                                         : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
           acc[t].x = fmaf(a, h.x, acc[t].x);
           acc[t].y = fmaf(a, h.y, acc[t].y);
           acc[t].z = fmaf(a, h.z, acc[t].z);
@@ -684,7 +691,7 @@ __global__ void __launch_bounds__(256)
     if (active) {
 #pragma unroll
       for (int t = 0; t < T; t++)
-        if (ok[t]) *reinterpret_cast<float4*>(Tout + j * r + 4 * (sub + LPR * t)) = acc[t];
+        if (FULL || ok[t]) *reinterpret_cast<float4*>(Tout + j * r + 4 * (sub + LPR * t)) = acc[t];
     }
   }
 }
@@ -835,6 +842,13 @@ template <class F>
 static int dispatch_gather(int r, bool aligned16, F&& f) {
   if (r % 4 == 0 && aligned16) {
     const int r4 = r / 4;
+    if (r4 == 4) return f(TypeTag<GatherVec4<4, 1, true>>{});
+    if (r4 == 8) return f(TypeTag<GatherVec4<8, 1, true>>{});
+    if (r4 == 16) return f(TypeTag<GatherVec4<16, 1, true>>{});
+    if (r4 == 32) return f(TypeTag<GatherVec4<32, 1, true>>{});
+    if (r4 == 64) return f(TypeTag<GatherVec4<64, 1, true>>{});
+    if (r4 == 128) return f(TypeTag<GatherVec4<64, 2, true>>{});
+    if (r4 == 256) return f(TypeTag<GatherVec4<64, 4, true>>{});
     if (r4 <= 4) return f(TypeTag<GatherVec4<4, 1>>{});
     if (r4 <= 8) return f(TypeTag<GatherVec4<8, 1>>{});
     if (r4 <= 16) return f(TypeTag<GatherVec4<16, 1>>{});
@@ -899,25 +913,26 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
                                int slots) {
   DN_CHECK(spmm_n_sweep_supported(r), "swept panels at rank %d", r);
   DN_CHECK(A->sweep_progress != nullptr, "matrix has no sweep counters");
-  sweep_kernel_t kernel = nullptr;
-  switch (r / 4 * 2 + (aligned ? 1 : 0)) {
-    case 8 * 2 + 1: kernel = k_spmm_n_sweep<8, true>; break;
-    case 8 * 2: kernel = k_spmm_n_sweep<8, false>; break;
-    case 16 * 2 + 1: kernel = k_spmm_n_sweep<16, true>; break;
-    case 16 * 2: kernel = k_spmm_n_sweep<16, false>; break;
-    case 32 * 2 + 1: kernel = k_spmm_n_sweep<32, true>; break;
-    case 32 * 2: kernel = k_spmm_n_sweep<32, false>; break;
-    case 64 * 2 + 1: kernel = k_spmm_n_sweep<64, true>; break;
-    default: kernel = k_spmm_n_sweep<64, false>; break;
+  static const sweep_kernel_t kernels[8] = {
+      k_spmm_n_sweep<8, false>,  k_spmm_n_sweep<8, true>,  k_spmm_n_sweep<16, false>,
+      k_spmm_n_sweep<16, true>,  k_spmm_n_sweep<32, false>, k_spmm_n_sweep<32, true>,
+      k_spmm_n_sweep<64, false>, k_spmm_n_sweep<64, true>};
+  static int kernel_regs[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // 0: attributes not yet set
+  const int variant = (r == 32 ? 0 : r == 64 ? 2 : r == 128 ? 4 : 6) + (aligned ? 1 : 0);
+  const sweep_kernel_t kernel = kernels[variant];
+  if (kernel_regs[variant] == 0) {
+    hipFuncAttributes attr;
+    DN_HIP(hipFuncGetAttributes(&attr, (const void*)kernel));
+    DN_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               SWEEP_LDS_BYTES));
+    kernel_regs[variant] = attr.numRegs > 0 ? attr.numRegs : 1;
   }
-  hipFuncAttributes attr;
-  DN_HIP(hipFuncGetAttributes(&attr, (const void*)kernel));
-  const int regs = (attr.numRegs + 7) / 8 * 8;
+  const int regs = (kernel_regs[variant] + 7) / 8 * 8;
   // two workgroups per CU: a workgroup puts waves / 4 waves on each of the 4 SIMDs
   int max_waves = SWEEP_REGISTER_BUDGET / (regs > 0 ? regs : 8) * 4 / 2;
   if (max_waves > 14) max_waves = 14;
   max_waves &= ~1;
-  DN_CHECK(max_waves >= 2, "the sweep kernel needs %d registers", attr.numRegs);
+  DN_CHECK(max_waves >= 2, "the sweep kernel needs %d registers", kernel_regs[variant]);
   const sweep_shape sh = sweep_shape_for(A->n_rows, r, max_waves);
   DN_CHECK(sh.waves > 0, "no sweep shape for rank %d", r);
   const int32_t* swept = A->panel_ids + A->n_plain;
@@ -926,8 +941,6 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
   if (const char* e = getenv("DNPEFF_SWEEP_SPIN")) spin_max = atoi(e);
   if (lag < 0) lag = 0;
   const size_t lds = sizeof(float) * (size_t)sh.rows_wg * r;
-  DN_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                             SWEEP_LDS_BYTES));
   for (int64_t pass = 0; pass < sh.n_pass; pass++) {
     const int64_t row0 = pass * sh.rows_per_pass;
     const int64_t row1 = row0 + sh.rows_per_pass < A->n_rows ? row0 + sh.rows_per_pass : A->n_rows;
@@ -1036,9 +1049,18 @@ int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_m
   if (grouped) {
     dim3 gg((unsigned)ceil_div(A->n_cols, 4 * SPMM_T_COLS));
     const int r4 = r / 4;
-#define DN_GROUPED(LPR, T)                                                                     \
-  hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T>), gg, block, 0, stream(), A->colptr, A->rowind, \
-                     A->tvals, A->n_cols, r, W_nr, T_mr, w_small)
+#define DN_GROUPED2(LPR, T, FULL, SMALL)                                                       \
+  hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T, FULL, SMALL>), gg, block, 0, stream(), A->colptr, \
+                     A->rowind, A->tvals, A->n_cols, r, W_nr, T_mr)
+#define DN_GROUPED(LPR, T)                                     \
+  do {                                                         \
+    const bool full = r == 4 * LPR * T;                        \
+    if (full && w_small24) DN_GROUPED2(LPR, T, true, true);    \
+    else if (full) DN_GROUPED2(LPR, T, true, false);           \
+    else if (w_small24) DN_GROUPED2(LPR, T, false, true);      \
+    else DN_GROUPED2(LPR, T, false, false);                    \
+  } while (0)
+    const bool w_small24 = w_small && A->n_rows < ((int64_t)1 << 24);
     if (r4 <= 4) DN_GROUPED(4, 1);
     else if (r4 <= 8) DN_GROUPED(8, 1);
     else if (r4 <= 16) DN_GROUPED(16, 1);
@@ -1046,6 +1068,7 @@ int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_m
     else if (r4 <= 64) DN_GROUPED(64, 1);
     else if (r4 <= 128) DN_GROUPED(64, 2);
     else DN_GROUPED(64, 4);
+#undef DN_GROUPED2
 #undef DN_GROUPED
   }
   dispatch_gather(width, aligned, [&](auto tag) {
