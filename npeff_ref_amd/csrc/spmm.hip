@@ -274,12 +274,15 @@ __global__ void __launch_bounds__(256)
 // the count says that all have finished piece i - 1 - lag.  The counter is only used by
 // workgroups of one XCD, which share an L2, so it is bumped and polled with L2 atomics of
 // workgroup scope (device scope costs a trip to the memory side per poll).  The wait is bounded
-// (spin_max polls): a grid that is not resident as a whole is slow but ends, and the sums do not
-// depend on the counter.  One partial sum per (row, XCD): part[row, slot0 + x, :].
+// (spin_max polls) and the first wait that runs out ends all later ones on that XCD (such a
+// workgroup adds SWEEP_GIVE_UP = 2^22, far above any count waited for; the few workgroups that
+// run out together each add it once: the grid has 64 per XCD), so a grid that is not resident
+// as a whole loses the lock step but not much time, and the sums do not depend on the counter.  One partial sum per (row, XCD): part[row, slot0 + x, :].
 // ---------------------------------------------------------------------------
 constexpr int SWEEP_SYNC_STRIDE = 32;    // ints between the progress counters of two XCDs
 constexpr int SWEEP_LDS_BYTES = 81920;   // running sums of a workgroup: half the LDS of a CU
 constexpr int SWEEP_MAX_SEGS = 32;       // rows per wave (their offsets live in the 64 lanes)
+constexpr int SWEEP_GIVE_UP = 1 << 22;   // added to a progress counter: every later wait ends at once
 
 template <int LPR, bool A16>
 __global__ void __launch_bounds__(1024)
@@ -353,13 +356,18 @@ __global__ void __launch_bounds__(1024)
       if (i == 0 && pi > lag) {
         if (threadIdx.x == 0) {
           const int want = (int)nq * (pi - lag);
-          for (int spin = 0; spin < spin_max; spin++) {
+          int spin = 0;
+          for (; spin < spin_max; spin++) {
             // an L2 atomic that changes nothing (the counter is never negative) reads the counter
             if (__hip_atomic_fetch_max(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >=
                 want)
               break;
             __builtin_amdgcn_s_sleep(8);
           }
+          // waited in vain (part of the grid is not running): nobody on this XCD waits again
+          if (spin == spin_max)
+            __hip_atomic_fetch_add(counter, SWEEP_GIVE_UP, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
         }
         __syncthreads();
       }

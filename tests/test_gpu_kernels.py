@@ -345,6 +345,11 @@ def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, monkeypa
     view = types.SimpleNamespace(ptr=ctypes.c_void_p(shifted.ptr.value + 4))
     d.op_spmm_n(A, r, view, dN)
     assert (np.abs(dN.numpy() - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
+    # workgroups that stop waiting for each other after one poll: same bits
+    monkeypatch.setenv("DNPEFF_SWEEP_SPIN", "1")
+    d.op_spmm_n(A, r, dH, dN)
+    assert np.array_equal(dN.numpy(), N)
+    monkeypatch.delenv("DNPEFF_SWEEP_SPIN")
     # without sweeps: every panel one wave per (row, panel) segment
     monkeypatch.setenv("DNPEFF_SWEEP_BYTES", "0")
     d.op_spmm_n(A, r, dH, dN)
