@@ -566,13 +566,17 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
   S->n_plain = n_plain;
   S->n_swept = n_swept;
   S->plan = plan;
+  if (getenv("DNPEFF_VERBOSE"))
+    fprintf(stderr, "dnpeff: %d column panels: %d plain, %d cut into %d swept pieces\n", P0, n_plain,
+            P0 - n_plain, n_swept);
   dfree(S->partials); S->partials = nullptr; S->partials_floats = 0;
   return 0;
 }
 
 // Panels pay when the gathered factor [n_cols, r] is far larger than the caches and there are
-// rows enough to share a panel's part of it: one coarse panel per ~48 MB of the factor, 8..512,
-// and few enough for the (panel, 4 rows) workgroups to fit one launch.  On 10,000 x 65.9M,
+// rows enough to share a panel's part of it: one coarse panel per ~48 MB of the factor, 8..512
+// (per ~96 MB, 8..256, at the ranks that have swept pieces), and few enough for the (panel, 4
+// rows) workgroups to fit one launch.  On 10,000 x 65.9M,
 // r = 128 (33.7 GB factor): no panels 29.3 ms, 32: 27.8, 128: 23.9, 256: 21.8, 512: 20.1 ms for
 // the gathers, plus 0.1 to 0.8 ms for the sum over panels; 1024 gains 1.1 ms and loses 0.7.
 // DNPEFF_PANELS overrides the number (0 = none).  Swept pieces hold DNPEFF_SWEEP_BYTES of the
@@ -581,9 +585,14 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
 static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   int64_t P = 0;
   const double bytes = 4.0 * (double)S->n_cols * r;
+  bool sweeps = spmm_n_sweep_supported(r);
+  if (const char* e = getenv("DNPEFF_SWEEP_BYTES")) sweeps = sweeps && atof(e) > 0.0;
   if (bytes >= 512e6 && S->n_rows >= 64) {
-    P = (int64_t)ceil(bytes / 48e6);
+    // with swept pieces for the panels in between, half as many coarse panels do as well for the
+    // gathers and halve the sum over the panels (configs[1]: 19.8 -> 19.4 ms for both)
+    P = (int64_t)ceil(bytes / (sweeps ? 96e6 : 48e6));
     if (P < 8) P = 8;
+    if (P > (sweeps ? 256 : 512)) P = sweeps ? 256 : 512;
   }
   if (const char* e = getenv("DNPEFF_PANELS")) P = atoi(e);
   if (P > 512) P = 512;
@@ -592,7 +601,7 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   if (P < 2 || S->nnz == 0) P = 0;
   panel_plan plan;
   plan.coarse = (int)P;
-  if (P > 0 && spmm_n_sweep_supported(r)) {
+  if (P > 0 && sweeps) {
     double sweep_bytes = 3.0 * 1024 * 1024;
     if (const char* e = getenv("DNPEFF_SWEEP_BYTES")) sweep_bytes = atof(e);
     if (sweep_bytes > 1e9) sweep_bytes = 1e9;  // (the kernel addresses a piece with 32 bits)
