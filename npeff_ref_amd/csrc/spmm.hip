@@ -264,9 +264,11 @@ __global__ void __launch_bounds__(256)
 // one after the other: LPR = r / 4 lanes gather one row of H with 16-byte loads, the 64 / LPR
 // lane groups take the entries of the segment round-robin and are added in a fixed butterfly
 // order before the segment's sum goes to LDS.  The (column, value) pairs of a segment are
-// requested two segments ahead and the segment offsets of a piece two pieces ahead, both right
-// after a batch of gathers has been issued: loads return in order, so a request from HBM placed
-// before gathers would hold those up.
+// requested two segments ahead, after the first gathers of a segment have been summed, and the
+// segment bounds of a piece two pieces ahead, at the end of a piece (before the wait for the
+// other workgroups): loads return in order, so a request from HBM placed before gathers holds
+// their results up.  Rows of H are addressed as the piece's first row plus a 32-bit offset (one
+// 24-bit multiply-add per gathered row), the pairs as a uniform base plus the lane.
 //
 // The workgroups of an XCD keep within `lag` pieces of each other: workgroups that ran ahead
 // (their rows hold fewer entries) would otherwise widen the part of H in use beyond the L2.
@@ -277,7 +279,8 @@ __global__ void __launch_bounds__(256)
 // (spin_max polls) and the first wait that runs out ends all later ones on that XCD (such a
 // workgroup adds SWEEP_GIVE_UP = 2^22, far above any count waited for; the few workgroups that
 // run out together each add it once: the grid has 64 per XCD), so a grid that is not resident
-// as a whole loses the lock step but not much time, and the sums do not depend on the counter.  One partial sum per (row, XCD): part[row, slot0 + x, :].
+// as a whole loses the lock step but not much time, and the sums do not depend on the counter.
+// One partial sum per (row, XCD): part[row, slot0 + x, :].
 // ---------------------------------------------------------------------------
 constexpr int SWEEP_SYNC_STRIDE = 32;    // ints between the progress counters of two XCDs
 constexpr int SWEEP_LDS_BYTES = 81920;   // running sums of a workgroup: half the LDS of a CU
