@@ -318,6 +318,7 @@ def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
     (32, 333, 5000, 300, 5, 200 * 128, 2),
     (256, 90, 2000, 700, 2, 400 * 1024, 8),      # 6 pieces: two XCDs have none
     (128, 40, 50000, 300, 16, 1000 * 512, 8),
+    (128, 40, 50000, 300, 16, 4 * 512, 8),       # more pieces than the split handles: fewer panels get cut
 ])
 def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, monkeypatch):
     """Coarse panels cut into L2-sized pieces that one XCD sweeps for all rows, running sums in

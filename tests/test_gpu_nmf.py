@@ -210,12 +210,13 @@ def test_column_panel_run_matches_oracle(monkeypatch):
     A.close()
 
 
-@pytest.mark.parametrize("r,waves", [(128, 14), (64, 3)])
-def test_swept_piece_run_matches_oracle(r, waves, monkeypatch):
-    """Column panels cut into small pieces that the XCDs sweep (forced on: 40 columns per piece,
-    any density): 50 iterations stay within the bar, and a second run gives the same bits."""
+@pytest.mark.parametrize("r,waves,piece_cols", [(128, 14, 40), (64, 3, 2000)])
+def test_swept_piece_run_matches_oracle(r, waves, piece_cols, monkeypatch):
+    """Column panels cut into small pieces that the XCDs sweep (forced on, any density; at 40
+    columns per piece all 6 panels are cut, at 2000 the 3 narrow ones stay whole and both kernels
+    share the product): 50 iterations stay within the bar, and a second run gives the same bits."""
     monkeypatch.setenv("DNPEFF_PANELS", "6")
-    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", str(40 * 4 * r))
+    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", str(piece_cols * 4 * r))
     monkeypatch.setenv("DNPEFF_SWEEP_MIN", "0")
     monkeypatch.setenv("DNPEFF_SWEEP_WAVES", str(waves))
     nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(300, 40000, 2048, r, 1e-8, 50, seed=9)
