@@ -946,6 +946,15 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
   DN_CHECK(max_waves >= 2, "the sweep kernel needs %d registers", kernel_regs[variant]);
   const sweep_shape sh = sweep_shape_for(A->n_rows, r, max_waves);
   DN_CHECK(sh.waves > 0, "no sweep shape for rank %d", r);
+  static bool told = false;
+  if (!told && getenv("DNPEFF_VERBOSE")) {
+    told = true;
+    fprintf(stderr,
+            "dnpeff: sweep kernel with %d registers: %lld workgroups of %d waves, %d rows each, "
+            "%lld pass(es) of %lld rows\n",
+            kernel_regs[variant], (long long)sh.wgs, sh.waves, sh.rows_wg, (long long)sh.n_pass,
+            (long long)sh.rows_per_pass);
+  }
   const int32_t* swept = A->panel_ids + A->n_plain;
   int lag = 0, spin_max = 400;
   if (const char* e = getenv("DNPEFF_SWEEP_LAG")) lag = atoi(e);
