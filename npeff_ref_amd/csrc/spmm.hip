@@ -12,6 +12,7 @@
 
 #include <cstdlib>
 #include <type_traits>
+#include <utility>
 
 namespace dn {
 
@@ -282,6 +283,17 @@ __global__ void __launch_bounds__(256)
 // as a whole loses the lock step but not much time, and the sums do not depend on the counter.
 // One partial sum per (row, XCD): part[row, slot0 + x, :].
 // ---------------------------------------------------------------------------
+// Every lane of a row of 16 lanes reads lane K of that row (DPP row_newbcast).
+template <int K>
+__device__ inline int row_bcast(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, 0x150 + K, 0xf, 0xf, true);
+}
+// f(integral_constant<int, I>) for I = 0 .. n - 1, unrolled at compile time
+template <class F, int... I>
+__device__ inline void each_step(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+
 constexpr int SWEEP_SYNC_STRIDE = 32;    // ints between the progress counters of two XCDs
 constexpr int SWEEP_LDS_BYTES = 81920;   // running sums of a workgroup: half the LDS of a CU
 constexpr int SWEEP_MAX_SEGS = 32;       // rows per wave (their offsets live in the 64 lanes)
@@ -386,20 +398,11 @@ __global__ void __launch_bounds__(1024)
       // that row with weight 0
       int my_i = lane < len ? ri - c0 : 0;
       float my_v = lane < len ? rv : 0.0f;
-      auto gathers = [&](auto u_tag, int st, float4* h, float* a) {
-        constexpr int U = decltype(u_tag)::value;
-#pragma unroll
-        for (int uu = 0; uu < U; uu++) {
-          const int u = ((st + uu) * G + grp) & 63;
-          a[uu] = __shfl(my_v, u);
-          const unsigned at = __umul24((unsigned)__shfl(my_i, u), r4) + sub16;
-          const float* hx = reinterpret_cast<const float*>(Hp + at);
-          if (A16) {
-            h[uu] = *reinterpret_cast<const float4*>(hx);
-          } else {
-            h[uu] = make_float4(hx[0], hx[1], hx[2], hx[3]);
-          }
-        }
+      auto gather_at = [&](int j) -> float4 {
+        const unsigned at = __umul24((unsigned)j, r4) + sub16;
+        const float* hx = reinterpret_cast<const float*>(Hp + at);
+        if (A16) return *reinterpret_cast<const float4*>(hx);
+        return make_float4(hx[0], hx[1], hx[2], hx[3]);
       };
       auto sums_up = [&](auto u_tag, const float4* h, const float* a) {
         constexpr int U = decltype(u_tag)::value;
@@ -413,47 +416,116 @@ __global__ void __launch_bounds__(1024)
       };
       using U2 = std::integral_constant<int, 2>;
       using U4 = std::integral_constant<int, 4>;
-      // the first gathers of the segment and their sums, then the request for the segment
-      // after the next
-      int nsteps = ((len < 64 ? len : 64) + G - 1) / G;
-      int st;
-      if (nsteps > 2) {
-        float4 h[4];
-        float a[4];
-        gathers(U4{}, 0, h, a);
-        sums_up(U4{}, h, a);
-        st = 4;
-      } else {
-        float4 h[2];
-        float a[2];
-        gathers(U2{}, 0, h, a);
-        sums_up(U2{}, h, a);
-        st = 2;
-      }
-      ri = pc2[lane];
-      rv = pv2[lane];
-      for (int base = 0; base < len; base += 64) {
-        if (base > 0) {
-          my_i = (pcol + s0)[base + lane];
-          my_v = (pval + s0)[base + lane];
-          my_i = base + lane < len ? my_i - c0 : 0;
-          my_v = base + lane < len ? my_v : 0.0f;
-          nsteps = ((len - base < 64 ? len - base : 64) + G - 1) / G;
-          st = 0;
+      if constexpr (LPR >= 16) {
+        // A lane group is one or more rows of 16 lanes.  One shuffle per 16 steps puts the pair
+        // of step 16 s + k of a lane's group into lane k of its row; each step then takes its
+        // pair with a row broadcast (a DPP operand, no LDS traffic): shuffles through the LDS
+        // crossbar for every step kept that pipe busy 68 % of the time.
+        const int row_lane = (lane & 15) * G + grp;
+        auto arrange = [&](int s, int& ai, float& av) {
+          const int src = (16 * G * s + row_lane) & 63;
+          ai = __shfl(my_i, src);
+          av = __shfl(my_v, src);
+        };
+        auto chunk = [&](auto st_tag, auto u_tag, int ai, float av) {
+          constexpr int ST = decltype(st_tag)::value;
+          constexpr int U = decltype(u_tag)::value;
+          float4 h[U];
+          float a[U];
+          each_step(std::make_integer_sequence<int, U>{}, [&](auto uu_tag) {
+            constexpr int uu = decltype(uu_tag)::value;
+            a[uu] = __int_as_float(row_bcast<ST + uu>(__float_as_int(av)));
+            h[uu] = gather_at(row_bcast<ST + uu>(ai));
+          });
+          sums_up(u_tag, h, a);
+        };
+        auto from = [&](auto st_tag, int n_s, int ai, float av) {  // steps ST .. of a sub-batch
+          constexpr int ST = decltype(st_tag)::value;
+          if (n_s - ST > 2) chunk(st_tag, U4{}, ai, av);
+          else chunk(st_tag, U2{}, ai, av);
+        };
+        auto after_first = [&](int n_s, int ai, float av) {
+          if (n_s > 4) from(std::integral_constant<int, 4>{}, n_s, ai, av);
+          if (n_s > 8) from(std::integral_constant<int, 8>{}, n_s, ai, av);
+          if (n_s > 12) from(std::integral_constant<int, 12>{}, n_s, ai, av);
+        };
+        int n_b = ((len < 64 ? len : 64) + G - 1) / G;  // steps of the batch
+        int ai;
+        float av;
+        arrange(0, ai, av);
+        // the first gathers of the segment and their sums (an empty segment gathers the piece's
+        // first row twice with weight 0), then the request for the segment after the next
+        from(std::integral_constant<int, 0>{}, n_b < 16 ? n_b : 16, ai, av);
+        ri = pc2[lane];
+        rv = pv2[lane];
+        after_first(n_b < 16 ? n_b : 16, ai, av);
+        for (int base = 0; base < len; base += 64) {
+          if (base > 0) {
+            my_i = (pcol + s0)[base + lane];
+            my_v = (pval + s0)[base + lane];
+            my_i = base + lane < len ? my_i - c0 : 0;
+            my_v = base + lane < len ? my_v : 0.0f;
+            n_b = ((len - base < 64 ? len - base : 64) + G - 1) / G;
+          }
+          for (int sb = base > 0 ? 0 : 1; 16 * sb < n_b; sb++) {
+            const int n_s = n_b - 16 * sb < 16 ? n_b - 16 * sb : 16;
+            arrange(sb, ai, av);
+            from(std::integral_constant<int, 0>{}, n_s, ai, av);
+            after_first(n_s, ai, av);
+          }
         }
-        while (st < nsteps) {
-          if (nsteps - st > 2) {
-            float4 h[4];
-            float a[4];
-            gathers(U4{}, st, h, a);
-            sums_up(U4{}, h, a);
-            st += 4;
-          } else {
-            float4 h[2];
-            float a[2];
-            gathers(U2{}, st, h, a);
-            sums_up(U2{}, h, a);
-            st += 2;
+      } else {
+        auto gathers = [&](auto u_tag, int st, float4* h, float* a) {
+          constexpr int U = decltype(u_tag)::value;
+#pragma unroll
+          for (int uu = 0; uu < U; uu++) {
+            const int u = ((st + uu) * G + grp) & 63;
+            a[uu] = __shfl(my_v, u);
+            h[uu] = gather_at(__shfl(my_i, u));
+          }
+        };
+        // the first gathers of the segment and their sums, then the request for the segment
+        // after the next
+        int nsteps = ((len < 64 ? len : 64) + G - 1) / G;
+        int st;
+        if (nsteps > 2) {
+          float4 h[4];
+          float a[4];
+          gathers(U4{}, 0, h, a);
+          sums_up(U4{}, h, a);
+          st = 4;
+        } else {
+          float4 h[2];
+          float a[2];
+          gathers(U2{}, 0, h, a);
+          sums_up(U2{}, h, a);
+          st = 2;
+        }
+        ri = pc2[lane];
+        rv = pv2[lane];
+        for (int base = 0; base < len; base += 64) {
+          if (base > 0) {
+            my_i = (pcol + s0)[base + lane];
+            my_v = (pval + s0)[base + lane];
+            my_i = base + lane < len ? my_i - c0 : 0;
+            my_v = base + lane < len ? my_v : 0.0f;
+            nsteps = ((len - base < 64 ? len - base : 64) + G - 1) / G;
+            st = 0;
+          }
+          while (st < nsteps) {
+            if (nsteps - st > 2) {
+              float4 h[4];
+              float a[4];
+              gathers(U4{}, st, h, a);
+              sums_up(U4{}, h, a);
+              st += 4;
+            } else {
+              float4 h[2];
+              float a[2];
+              gathers(U2{}, st, h, a);
+              sums_up(U2{}, h, a);
+              st += 2;
+            }
           }
         }
       }
