@@ -734,12 +734,13 @@ __global__ void __launch_bounds__(256)
                                                 (__umul24((unsigned)jrow, r4) + sub16));
         return W + (int64_t)jrow * r + 4 * sub;
       };
-      int u = 0;
-      for (; u + UNR <= cmax; u += UNR) {
-        float4 h[UNR][T];
-        float a[UNR];
+      // U entries of every group with their gathers in flight together
+      auto block = [&](auto u_tag, int u) {
+        constexpr int U = decltype(u_tag)::value;
+        float4 h[U][T];
+        float a[U];
 #pragma unroll
-        for (int uu = 0; uu < UNR; uu++) {
+        for (int uu = 0; uu < U; uu++) {
           const float* x = wrow(__shfl(my_i, gbase + u + uu));
           a[uu] = __shfl(my_v, gbase + u + uu);
 #pragma unroll
@@ -748,7 +749,7 @@ __global__ void __launch_bounds__(256)
                                      : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
-        for (int uu = 0; uu < UNR; uu++)
+        for (int uu = 0; uu < U; uu++)
 #pragma unroll
           for (int t = 0; t < T; t++) {
             acc[t].x = fmaf(a[uu], h[uu][t].x, acc[t].x);
@@ -756,19 +757,17 @@ __global__ void __launch_bounds__(256)
             acc[t].z = fmaf(a[uu], h[uu][t].z, acc[t].z);
             acc[t].w = fmaf(a[uu], h[uu][t].w, acc[t].w);
           }
-      }
-      for (; u < cmax; u++) {
-        const float* x = wrow(__shfl(my_i, gbase + u));
-        const float a = __shfl(my_v, gbase + u);
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-          const float4 h = FULL || ok[t] ? *reinterpret_cast<const float4*>(x + 4 * LPR * t)
-                                         : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          acc[t].x = fmaf(a, h.x, acc[t].x);
-          acc[t].y = fmaf(a, h.y, acc[t].y);
-          acc[t].z = fmaf(a, h.z, acc[t].z);
-          acc[t].w = fmaf(a, h.w, acc[t].w);
-        }
+      };
+      int u = 0;
+      for (; u + UNR <= cmax; u += UNR) block(std::integral_constant<int, UNR>{}, u);
+      // what is left, also in one go: most columns hold one to three entries, and one at a time
+      // each of them would wait for its own round trip
+      if constexpr (UNR == 4) {
+        if (cmax - u == 3) block(std::integral_constant<int, 3>{}, u);
+        else if (cmax - u == 2) block(std::integral_constant<int, 2>{}, u);
+        else if (cmax - u == 1) block(std::integral_constant<int, 1>{}, u);
+      } else if constexpr (UNR == 2) {
+        if (cmax - u == 1) block(std::integral_constant<int, 1>{}, u);
       }
     }
     if (active) {
