@@ -319,6 +319,9 @@ def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
     (256, 90, 2000, 700, 2, 400 * 1024, 8),      # 6 pieces: two XCDs have none
     (128, 40, 50000, 300, 16, 1000 * 512, 8),
     (128, 40, 50000, 300, 16, 4 * 512, 8),       # more pieces than the split handles: fewer panels get cut
+    (64, 200, 4000, 3000, 2, 300 * 256, 8),      # long segments at 4 lane groups (several batches of 64)
+    (32, 150, 3000, 2500, 2, 400 * 128, 4),      # long segments at 8 lane groups (shuffles, no row broadcasts)
+    (256, 120, 3000, 2800, 2, 500 * 1024, 6),    # long segments at one lane group (4 rows of 16 lanes)
 ])
 def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, monkeypatch):
     """Coarse panels cut into L2-sized pieces that one XCD sweeps for all rows, running sums in
