@@ -322,6 +322,17 @@ int dnpeff_topk_rows(int64_t n_rows, int64_t count, int64_t k, const float* x, f
 /* G[r, r] = X^T X for X [rows, r].  cublasSgemm at device_contexts1.h:303,322. */
 int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr);
 
+/* The same product for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the
+ * reference.  The slice partials that dnpeff_op_gram keeps in a buffer it allocates go to a
+ * static 8 MiB device array instead; the call allocates and frees nothing and does not wait for
+ * the device (call dnpeff_sync() before reading G).  Limits: 1 <= r <= 128; any number of rows at
+ * r <= 32, at most 52,224 rows above (a larger request is refused with an error).  Same kernels,
+ * same summation order, same bits as dnpeff_op_gram.  All calls on one GPU share the array:
+ * calls queued on the library stream run one after the other, calls that overlap on one GPU
+ * (other threads, other streams) race. */
+int dnpeff_op_gram_static(int64_t rows, int r, const float* X, float* G_rr);
+
 /* out = X * num / (X G + eps) with X, num, out [rows, r], G [r, r] symmetric.
  * out may alias num but not X.  D_out (may be NULL) receives X G.
  * cublasSgemm + kernelNmfMuUpdate at device_contexts1.h:306-308,329-332. */

@@ -33,6 +33,7 @@ from .binding import (  # noqa: F401
     topk_rows,
     op_spmm_t,
     op_gram,
+    op_gram_static,
     op_xg_mu,
     op_xg_mu_gram,
     op_dot,

@@ -100,6 +100,7 @@ SIGNATURES = {
     "dnpeff_op_spmm_n": (C.c_int, [_p, C.c_int, _p, _p]),
     "dnpeff_op_spmm_t": (C.c_int, [_p, C.c_int, _p, _p]),
     "dnpeff_op_gram": (C.c_int, [_i64, C.c_int, _p, _p]),
+    "dnpeff_op_gram_static": (C.c_int, [_i64, C.c_int, _p, _p]),
     "dnpeff_op_xg_mu": (C.c_int, [_i64, C.c_int, _p, _p, _p, _f32, _p, _p]),
     "dnpeff_op_xg_mu_gram": (C.c_int, [_i64, _p, _p, _p, _f32, _p, _p]),
     "dnpeff_op_dot": (C.c_int, [_i64, _p, _p, C.POINTER(_f64)]),
@@ -221,6 +222,11 @@ def op_spmm_t(A: "Csr", r: int, W_nr: DeviceArray, T_mr: DeviceArray):
 
 def op_gram(X: DeviceArray, G: DeviceArray):
     _check(lib.dnpeff_op_gram(X.shape[0], X.shape[1], X.ptr, G.ptr))
+
+
+def op_gram_static(X: DeviceArray, G: DeviceArray, rows: Optional[int] = None):
+    """G = X^T X of the first `rows` rows of X through the entry point that allocates nothing."""
+    _check(lib.dnpeff_op_gram_static(X.shape[0] if rows is None else rows, X.shape[1], X.ptr, G.ptr))
 
 
 def op_xg_mu(X: DeviceArray, G: DeviceArray, num: DeviceArray, eps: float, out: DeviceArray, D_out=None):

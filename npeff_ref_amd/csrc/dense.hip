@@ -1861,6 +1861,50 @@ DN_API int dnpeff_op_gram(int64_t rows, int r, const float* X, float* G_rr) {
   return s;
 }
 
+// ---------------------------------------------------------------------------
+// The Gram product without any allocation: the slice partials go to a file-scope device array.
+// Every GPU holds its own copy of the array at its own address, taken once per device with
+// hipGetSymbolAddress; host code never uses the array's name as a pointer.
+// ---------------------------------------------------------------------------
+constexpr int64_t GRAM_STATIC_FLOATS = 2 * 1024 * 1024;  // 8 MiB per GPU, held until the process ends
+constexpr int GRAM_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[GRAM_STATIC_FLOATS];
+static float* g_scratch_ptr[GRAM_STATIC_MAX_DEVICES] = {};
+
+// Address of this device's copy of the scratch array (looked up on first use on a device).
+static int gram_static_scratch(float** out) {
+  int dev = 0;
+  DN_HIP(hipGetDevice(&dev));
+  DN_CHECK(dev >= 0 && dev < GRAM_STATIC_MAX_DEVICES, "device %d outside [0, %d)", dev,
+           GRAM_STATIC_MAX_DEVICES);
+  if (!g_scratch_ptr[dev]) {
+    float* p = nullptr;
+    DN_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+    DN_CHECK(p != nullptr, "no device address for the static scratch array");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+DN_API int dnpeff_op_gram_static(int64_t rows, int r, const float* X, float* G_rr) {
+  clear_error();
+  DN_CHECK(X && G_rr, "NULL argument");
+  DN_CHECK(rows >= 1, "rows must be at least 1 (got %lld)", (long long)rows);
+  DN_CHECK(r >= 1 && r <= 128, "dnpeff_op_gram_static handles ranks 1..128 (got %d)", r);
+  const int64_t need = gram_workspace_floats(rows, r);
+  DN_CHECK(need <= GRAM_STATIC_FLOATS,
+           "dnpeff_op_gram_static: %lld rows at rank %d need %lld floats of partial sums, the static "
+           "scratch holds %lld (at most %lld rows at ranks above 32)",
+           (long long)rows, r, (long long)need, (long long)GRAM_STATIC_FLOATS,
+           (long long)(GRAM_STATIC_FLOATS / (gram_pairs(128) * 1024) * 256));
+  float* ws = nullptr;
+  DN_TRY(gram_static_scratch(&ws));
+  // every partial block that the reduction reads is written by the product kernel of the same
+  // call, so nothing of the last call's contents needs clearing
+  return launch_gram(rows, r, X, G_rr, ws);
+}
+
 DN_API int dnpeff_op_xg_mu(int64_t rows, int r, const float* X, const float* G_rr, const float* num,
                            float eps, float* out, float* D_out) {
   clear_error();
