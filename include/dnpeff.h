@@ -56,6 +56,22 @@ int dnpeff_sync(void);
 /* Library stream as a hipStream_t, for callers that order their own work. */
 void* dnpeff_stream(void);
 
+/* Free and total memory of the current device in bytes (hipMemGetInfo); either pointer may be
+ * NULL.  The reference prints the same figures through NVML
+ * (cc/cuda_d_npeff/src/cuda/debugging/). */
+int dnpeff_device_memory(int64_t* free_bytes, int64_t* total_bytes);
+
+/* Switches for experiments and for tests that must reach a particular code path; no counterpart
+ * in the reference.  Names: dense_fill, panels, sweep_bytes, sweep_min, sweep_waves, sweep_lag,
+ * sweep_spin, spmm_t_slices, split_bf16, fused_gram, h_tile_mb, tiled_h, topk_fast_cap, verbose.
+ * Each starts from the environment variable DNPEFF_<NAME IN CAPITALS> (read once, when the
+ * library is first used) or its default; plans take the values when they are made
+ * (dnpeff_nmf_create, the first product on a matrix).  dnpeff_tuning_reset() goes back to the
+ * starting values.  An unknown name is an error. */
+int dnpeff_tuning_set(const char* name, double value);
+int dnpeff_tuning_get(const char* name, double* value);
+int dnpeff_tuning_reset(void);
+
 /* Plain device buffers for callers of the dnpeff_op_* entry points that have
  * no device allocator of their own (DeviceCudaContext::dmalloc / dfree and the
  * copies of cc/cuda_d_npeff/src/cuda/cuda_context.h:58-69, transfers.h).
@@ -132,7 +148,8 @@ int dnpeff_csr_build_transpose(dnpeff_csr* A);
  * is a multiple of 4.  dnpeff_csr_download and the loader calls still see the whole matrix;
  * any call that edits the matrix undoes the split.  The threshold is raised until both dense
  * blocks fit an eighth of the device memory.  min_fill <= 0 removes the split.  n_dense (may
- * be NULL) receives the number of columns in the head.
+ * be NULL) receives the number of columns in the head.  A matrix in which a row holds the same
+ * column twice is refused by the products (dnpeff_csr_build_transpose reports it).
  * No counterpart in the reference, which hands the whole matrix to cusparseSpMM
  * (device_contexts1.h:255-265); dnpeff_nmf_create applies it by itself (fill 1/16, rank >= 64
  * and a multiple of 4, at least 1024 rows) unless the caller has split the matrix already. */
@@ -198,6 +215,22 @@ float dnpeff_uniform_at(uint64_t seed, int matrix_id, int64_t row, int64_t col, 
  * multi_mu_dense_factors_device_contexts1.h:129-170,384-434).
  * Like the reference it refuses n_rows > n_cols. */
 int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out);
+
+/* The same with flags.  DNPEFF_NMF_CONSUME_MATRIX: the context may free every array of A that
+ * its products do not read (the caller's row-major arrays once the dense head, the transposed
+ * copy and the regrouped copy exist), as the reference's host matrix can be dropped once
+ * moveAToDeviceAsync has copied it (device_contexts1.h:182-195).  Afterwards A still answers
+ * dnpeff_csr_shape, dnpeff_csr_kept_indices and dnpeff_csr_full_dense_size and serves this and
+ * later contexts of the same rank, but dnpeff_csr_download and the loader calls fail with an
+ * error.  This is what lets a matrix whose copies and factors fill the device fit.
+ * When a second [m, r] array does not fit beside H, the context updates H on column tiles
+ * (A^T W of a tile, then the tile's update) with the same results. */
+enum { DNPEFF_NMF_CONSUME_MATRIX = 1 };
+int dnpeff_nmf_create_ex(dnpeff_csr* A, int rank, float eps, int64_t seed, unsigned flags,
+                         dnpeff_nmf** out);
+
+/* Whether the context updates H on column tiles, and the tile width in columns (0 if not). */
+int dnpeff_nmf_info(const dnpeff_nmf* nmf, int* tiled, int64_t* tile_cols);
 
 /* W then H ~ U[0,1) from the seed (initializeW / initializeH,
  * multi_mu_dense_factors_device_contexts1.h:197-233). */

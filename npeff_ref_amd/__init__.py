@@ -27,6 +27,10 @@ from .binding import (  # noqa: F401
     KERNEL_CLASSES,
     sync,
     device_info,
+    device_memory,
+    tuning_set,
+    tuning_get,
+    tuning_reset,
     op_mu,
     op_spmm_n,
     op_threshold_compact,

@@ -45,6 +45,10 @@ SIGNATURES = {
     "dnpeff_device_info": (C.c_int, [C.c_char_p, C.c_int, C.POINTER(_i64), C.POINTER(C.c_int)]),
     "dnpeff_sync": (C.c_int, []),
     "dnpeff_stream": (_p, []),
+    "dnpeff_device_memory": (C.c_int, [C.POINTER(_i64), C.POINTER(_i64)]),
+    "dnpeff_tuning_set": (C.c_int, [C.c_char_p, _f64]),
+    "dnpeff_tuning_get": (C.c_int, [C.c_char_p, C.POINTER(_f64)]),
+    "dnpeff_tuning_reset": (C.c_int, []),
     "dnpeff_dev_malloc": (C.c_int, [_i64, _pp]),
     "dnpeff_dev_free": (C.c_int, [_p]),
     "dnpeff_dev_upload": (C.c_int, [_p, _p, _i64]),
@@ -75,6 +79,8 @@ SIGNATURES = {
     ),
     "dnpeff_uniform_at": (_f32, [_u64, C.c_int, _i64, _i64, _i64]),
     "dnpeff_nmf_create": (C.c_int, [_p, C.c_int, _f32, _i64, _pp]),
+    "dnpeff_nmf_create_ex": (C.c_int, [_p, C.c_int, _f32, _i64, C.c_uint, _pp]),
+    "dnpeff_nmf_info": (C.c_int, [_p, C.POINTER(C.c_int), C.POINTER(_i64)]),
     "dnpeff_nmf_init_factors": (C.c_int, [_p]),
     "dnpeff_nmf_set_factors": (C.c_int, [_p, _p, _p]),
     "dnpeff_nmf_step": (C.c_int, [_p, C.c_int]),
@@ -146,6 +152,27 @@ def device_info():
 
 def sync():
     _check(lib.dnpeff_sync())
+
+
+def device_memory():
+    """(free, total) bytes of device memory."""
+    f, t = _i64(0), _i64(0)
+    _check(lib.dnpeff_device_memory(C.byref(f), C.byref(t)))
+    return f.value, t.value
+
+
+def tuning_set(name: str, value: float):
+    _check(lib.dnpeff_tuning_set(name.encode(), float(value)))
+
+
+def tuning_get(name: str) -> float:
+    v = _f64(0)
+    _check(lib.dnpeff_tuning_get(name.encode(), C.byref(v)))
+    return v.value
+
+
+def tuning_reset():
+    _check(lib.dnpeff_tuning_reset())
 
 
 def size_of_split(total: int, n_splits: int, split_index: int) -> int:
@@ -437,14 +464,29 @@ class MuNmf:
     """Dense-factor multiplicative-update NMF on one GPU (MuNmf<IndT>,
     multi_mu_dense_factors_nmf1.h:42-375)."""
 
-    def __init__(self, A: Csr, params: MuNmfParams):
+    def __init__(self, A: Csr, params: MuNmfParams, consume_matrix: bool = False):
+        """consume_matrix: the context may free the arrays of A that its products do not read
+        (DNPEFF_NMF_CONSUME_MATRIX), for matrices that only fit the device that way."""
         self.A = A
         self.params = params
         self.n_rows, self.n_cols, _ = A._shape3()
         h = C.c_void_p()
-        _check(lib.dnpeff_nmf_create(A._h, params.rank, params.eps, params.seed, C.byref(h)))
+        _check(lib.dnpeff_nmf_create_ex(A._h, params.rank, params.eps, params.seed,
+                                        1 if consume_matrix else 0, C.byref(h)))
         self._h = h
         self._initialized = False
+
+    def info(self):
+        """(tiled H update?, tile width in columns)."""
+        t, c = C.c_int(0), _i64(0)
+        _check(lib.dnpeff_nmf_info(self._h, C.byref(t), C.byref(c)))
+        return bool(t.value), c.value
+
+    def device_factors(self):
+        """Device addresses of W [n, r] and H [m, r]."""
+        w, h = C.c_void_p(), C.c_void_p()
+        _check(lib.dnpeff_nmf_device_factors(self._h, C.byref(w), C.byref(h)))
+        return w.value, h.value
 
     def initialize(self):
         """_initializeBeforeRun (nmf1.h:128-150): W then H ~ U[0,1) from the seed."""

@@ -40,7 +40,7 @@ struct Profiler {
     if (!enabled) return 0;
     DN_HIP(hipEventRecord(pool[used].stop, stream()));
     used++;
-    if (used >= 4096) return collect();
+    if (used >= 32768) return collect();
     return 0;
   }
   int collect() {
@@ -81,8 +81,15 @@ struct dnpeff_nmf {
   float* W = nullptr;        // [n, r]
   float* W2 = nullptr;       // [n, r] output buffer of the W update
   float* Nw = nullptr;       // [n, r] A H^T
-  float* H = nullptr;        // [m, r]
-  float* S = nullptr;        // [m, r] A^T W, then the updated H
+  float* H = nullptr;        // [m, r] (points into Hbuf)
+  float* S = nullptr;        // [m, r] A^T W, then the updated H; tiled: [tile_cols, r], A^T W of a tile
+  float* Hbuf = nullptr;     // allocation that holds H; tiled: [m + tile_cols, r]
+  // Tiled H update (when a second [m, r] array does not fit): A^T W is formed for tile_cols
+  // columns at a time and the updated tile is written one tile below (or above) the place of the
+  // old one inside Hbuf, so the update needs no full-size output: H alternates between
+  // Hbuf and Hbuf + tile_cols r.
+  bool tiled = false;
+  int64_t tile_cols = 0;
   float* G = nullptr;        // [r, r]
   float* G2 = nullptr;       // [r, r]
   float* gram_ws = nullptr;  // slice partials of the Gram kernel
@@ -98,65 +105,176 @@ struct dnpeff_nmf {
 DN_API int dnpeff_nmf_destroy(dnpeff_nmf* nmf) {
   if (!nmf) return 0;
   (void)hipStreamSynchronize(stream());
-  dfree(nmf->W); dfree(nmf->W2); dfree(nmf->Nw); dfree(nmf->H); dfree(nmf->S);
+  dfree(nmf->W); dfree(nmf->W2); dfree(nmf->Nw); dfree(nmf->Hbuf); dfree(nmf->S);
   dfree(nmf->G); dfree(nmf->G2); dfree(nmf->gram_ws); dfree(nmf->dot_ws);
   dfree(nmf->GH); dfree(nmf->gpart);
   delete nmf;
   return 0;
 }
 
-// Splits off the dense head when the products can use it: rank a multiple of 4 and at least 64
-// (below that a column of the dense block costs more than its entries do as gathers), enough
-// rows for the fill fraction to mean something.  A column goes to the head when at least 1/16 of
-// the rows hold it; DNPEFF_DENSE_FILL overrides the fraction (0 = never split).
-static int default_head_split(dnpeff_csr* A, int rank) {
-  double fill = 1.0 / 16.0;
-  if (const char* e = getenv("DNPEFF_DENSE_FILL")) fill = atof(e);
-  if (A->tail) {
-    if (rank % 4 == 0) return 0;  // split by the caller: keep it
-    fill = 0.0;
-  }
-  if (fill <= 0.0 || fill > 1.0 || rank % 4 != 0 || rank < 64 || A->n_rows < 1024) {
-    if (A->tail) return dnpeff_csr_split_dense_head(A, 0.0, nullptr);
-    return 0;
-  }
-  return dnpeff_csr_split_dense_head(A, fill, nullptr);
-}
-
 // The H update also produces H^T H (one pass over H instead of two) when the rank is 128 and
-// the factor is large enough for the pass to matter.  DNPEFF_FUSED_GRAM=0 switches it off.
+// the factor is large enough for the pass to matter (fused_gram switch: 0 = off).
 static bool fused_update(const dnpeff_nmf* h) {
-  if (const char* e = getenv("DNPEFF_FUSED_GRAM"))
-    if (atoi(e) == 0) return false;
+  if (tuning().fused_gram == 0.0 || h->tiled) return false;
   return h->r == 128 && h->m >= 4096;
 }
 
-DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out) {
+// Columns of a tile of the tiled H update: h_tile_mb MiB of the factor, a multiple of 128.
+static int64_t tile_cols_for(int64_t m, int rank) {
+  double mb = tuning().h_tile_mb;
+  if (mb < 0.001) mb = 0.001;
+  int64_t t = (int64_t)(mb * 1024.0 * 1024.0 / (4.0 * rank)) / 128 * 128;
+  if (t < 128) t = 128;
+  const int64_t m_pad = ceil_div(m, 128) * 128;
+  return t < m_pad ? t : m_pad;
+}
+
+// Bytes of device memory that the handle allocates besides the structures of the matrix.
+static double factor_bytes(int64_t n, int64_t m, int rank, bool tiled) {
+  const double nr = 4.0 * (double)n * rank, mr = 4.0 * (double)m * rank;
+  double ws = (double)gram_workspace_floats(m, rank), ws_n = (double)gram_workspace_floats(n, rank);
+  if (ws_n > ws) ws = ws_n;
+  const double tile = 4.0 * (double)tile_cols_for(m, rank) * rank;
+  return 3.0 * nr + (tiled ? mr + 2.0 * tile : 2.0 * mr) + 4.0 * ws + 3.0 * 4.0 * rank * rank +
+         4.0 * (double)xg_mu_gram_workspace_floats(m);
+}
+
+// What the products' own buffers take besides the two sparse copies and the dense blocks: partial
+// sums of A H^T, segment offsets, column offsets, work lists, head workspace (upper estimates),
+// plus room that is left free.
+static double product_overhead_bytes(const dnpeff_csr* A, int rank) {
+  const double n = (double)A->n_rows, m = (double)A->n_cols;
+  double partials = 4.0 * rank * (double)A->nnz / (double)SPMM_N_CHUNK + 4.0 * rank * n;
+  if (partials < 3.2e9 && 4.0 * m * rank >= 512e6) partials = 3.2e9;
+  return partials + 8.0 * n * 3100.0 + 8.0 * m + 4.0 * m + 1.5e9 + 4.0e9;
+}
+
+// Splits off the dense head when the products can use it: rank a multiple of 4 and at least 64
+// (below that a column of the dense block costs more than its entries do as gathers), enough
+// rows for the fill fraction to mean something.  A column goes to the head when at least 1/16 of
+// the rows hold it (dense_fill switch; 0 = never split); the fraction is doubled until the dense
+// blocks and both sparse copies of the rest fit the memory left beside the factors.  *tiled
+// receives whether the H update must run on column tiles for everything to fit.
+static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
+  const tuning_t& tn = tuning();
+  size_t free_b = 0, total_b = 0;
+  DN_HIP(hipMemGetInfo(&free_b, &total_b));
+  const dnpeff_csr* S0 = sparse_part(A);
+  // memory that the matrix structures may take: what is free now, plus what a consuming create
+  // releases, plus what the structures hold already
+  double avail = (double)free_b;
+  if (consume && A->colind && A->vals) avail += 8.0 * (double)A->nnz;
+  if (A->tail) {
+    avail += 8.0 * (double)A->head.n_pad * (double)A->head.n_d_pad;
+    if (S0->colind) avail += 8.0 * (double)S0->nnz;
+  }
+  if (S0->colptr) avail += 8.0 * (double)S0->nnz;
+  if (S0->pcol) avail += 8.0 * (double)S0->nnz;
+  avail -= product_overhead_bytes(A, rank);
+  const double budget_full = avail - factor_bytes(A->n_rows, A->n_cols, rank, false);
+  const double budget_tiled = avail - factor_bytes(A->n_rows, A->n_cols, rank, true);
+  const bool can_split = rank % 4 == 0 && rank >= 64 && A->n_rows >= 1024;
+  double fill = tn.dense_fill;
+  if (fill > 1.0) fill = 0.0;
+  *tiled = tn.tiled_h > 0.0;
+  if (A->tail) {
+    if (rank % 4 == 0) {  // split by the caller (or an earlier handle): keep it
+      const double foot = 8.0 * (double)A->head.n_pad * (double)A->head.n_d_pad + 16.0 * (double)S0->nnz;
+      if (tn.tiled_h < 0.0) *tiled = foot > budget_full;
+      return 0;
+    }
+    DN_TRY(dnpeff_csr_split_dense_head(A, 0.0, nullptr));
+    fill = 0.0;
+  }
+  if (!can_split) fill = 0.0;
+  if (!has_row_major(A)) {  // consumed by an earlier handle without a head: nothing to choose
+    if (tn.tiled_h < 0.0) *tiled = 16.0 * (double)A->nnz > budget_full;
+    return 0;
+  }
+  head_choice c;
+  DN_TRY(choose_dense_head(A, fill, *tiled ? budget_tiled : budget_full, &c));
+  if (!c.fits && tn.tiled_h < 0.0 && !*tiled) {
+    *tiled = true;
+    DN_TRY(choose_dense_head(A, fill, budget_tiled, &c));
+  }
+  if (tn.verbose != 0.0)
+    fprintf(stderr,
+            "dnpeff: plan for rank %d: %.1f GB free, budget for the matrix %.1f GB (%s H update); dense "
+            "head of %lld columns (>= %lld entries), footprint %.1f GB%s\n",
+            rank, (double)free_b / 1e9, (*tiled ? budget_tiled : budget_full) / 1e9,
+            *tiled ? "tiled" : "full-size", (long long)c.n_d, (long long)c.thr, c.footprint / 1e9,
+            c.fits ? "" : " (over budget)");
+  if (c.thr == 0) return 0;  // no head (there is none to undo either)
+  return split_dense_head_at(A, c.thr, nullptr);
+}
+
+static int nmf_create_impl(dnpeff_csr* A, int rank, float eps, int64_t seed, unsigned flags,
+                           dnpeff_nmf** out) {
   clear_error();
   DN_CHECK(out != nullptr, "out is NULL");
   *out = nullptr;
   DN_CHECK(A != nullptr, "matrix is NULL");
   DN_CHECK(rank >= 1 && rank <= 1024, "rank %d outside [1, 1024]", rank);
+  DN_CHECK((flags & ~(unsigned)DNPEFF_NMF_CONSUME_MATRIX) == 0, "unknown flags 0x%x", flags);
   // multi_mu_dense_factors_nmf1.h:95-99
   DN_CHECK(A->n_rows <= A->n_cols, "Error: Not handling matrices with more rows than columns yet.");
-  DN_TRY(default_head_split(A, rank));
+  const bool consume = (flags & DNPEFF_NMF_CONSUME_MATRIX) != 0;
+  double sq_norm = 0.0;
+  DN_TRY(dnpeff_csr_sq_norm(A, &sq_norm));
+  bool tiled = false;
+  DN_TRY(plan_matrix(A, rank, consume, &tiled));
+  if (consume && A->tail) {  // the tail and the head hold everything the products read
+    DN_HIP(hipStreamSynchronize(stream()));
+    dfree(A->colind); A->colind = nullptr;
+    dfree(A->vals); A->vals = nullptr;
+  }
   DN_TRY(csr_ensure_products(A, rank));
+  if (consume) DN_TRY(csr_consume_for_products(A));
   dnpeff_nmf* h = new dnpeff_nmf();
   h->A = A; h->r = rank; h->eps = eps; h->seed = (uint64_t)seed;
   h->n = A->n_rows; h->m = A->n_cols;
+  h->sq_norm_A = sq_norm;
+  h->tiled = tiled && A->n_cols > 0;
+  h->tile_cols = h->tiled ? tile_cols_for(h->m, rank) : 0;
   const int64_t nr = h->n * rank, mr = h->m * rank;
+  const int64_t h_floats = h->tiled ? (h->m + h->tile_cols) * rank : mr;
+  const int64_t s_floats = h->tiled ? h->tile_cols * rank : mr;
   int64_t ws = gram_workspace_floats(h->m, rank);
   int64_t ws_n = gram_workspace_floats(h->n, rank);
   if (ws_n > ws) ws = ws_n;
   int s = dmalloc(&h->W, nr) || dmalloc(&h->W2, nr) || dmalloc(&h->Nw, nr) ||
-          dmalloc(&h->H, mr) || dmalloc(&h->S, mr) || dmalloc(&h->G, (int64_t)rank * rank) ||
-          dmalloc(&h->G2, (int64_t)rank * rank) || dmalloc(&h->gram_ws, ws) ||
-          dmalloc(&h->dot_ws, DOT_BLOCKS + 2);
+          dmalloc(&h->Hbuf, h_floats) || dmalloc(&h->S, s_floats) ||
+          dmalloc(&h->G, (int64_t)rank * rank) || dmalloc(&h->G2, (int64_t)rank * rank) ||
+          dmalloc(&h->gram_ws, ws) || dmalloc(&h->dot_ws, DOT_BLOCKS + 2);
+  h->H = h->Hbuf;
   if (!s && fused_update(h))
     s = dmalloc(&h->GH, (int64_t)rank * rank) || dmalloc(&h->gpart, xg_mu_gram_workspace_floats(h->m));
-  if (!s) s = dnpeff_csr_sq_norm(A, &h->sq_norm_A);
+  if (!s && h->tiled) s = csr_tile_lists(A);
   if (s) { dnpeff_nmf_destroy(h); return s; }
+  if (tuning().verbose != 0.0) {
+    size_t free_b = 0, total_b = 0;
+    (void)hipMemGetInfo(&free_b, &total_b);
+    fprintf(stderr, "dnpeff: factors allocated (%s H update%s), %.1f GB of %.1f GB left free\n",
+            h->tiled ? "tiled" : "full-size", consume ? ", matrix consumed" : "", (double)free_b / 1e9,
+            (double)total_b / 1e9);
+  }
   *out = h;
+  return 0;
+}
+
+DN_API int dnpeff_nmf_create(dnpeff_csr* A, int rank, float eps, int64_t seed, dnpeff_nmf** out) {
+  return nmf_create_impl(A, rank, eps, seed, 0u, out);
+}
+
+DN_API int dnpeff_nmf_create_ex(dnpeff_csr* A, int rank, float eps, int64_t seed, unsigned flags,
+                                dnpeff_nmf** out) {
+  return nmf_create_impl(A, rank, eps, seed, flags, out);
+}
+
+DN_API int dnpeff_nmf_info(const dnpeff_nmf* nmf, int* tiled, int64_t* tile_cols) {
+  DN_CHECK(nmf != nullptr, "handle is NULL");
+  if (tiled) *tiled = nmf->tiled ? 1 : 0;
+  if (tile_cols) *tile_cols = nmf->tile_cols;
   return 0;
 }
 
@@ -179,10 +297,25 @@ DN_API int dnpeff_nmf_set_factors(dnpeff_nmf* nmf, const float* W_nr, const floa
   if (H_rm) {
     nmf->gh_valid = false;
     nmf->nw_valid = false;
-    DN_HIP(hipMemcpy(nmf->S, H_rm, sizeof(float) * nmf->m * nmf->r, hipMemcpyHostToDevice));
-    DN_TRY(launch_transpose(nmf->r, nmf->m, nmf->S, nmf->H));
-    DN_HIP(hipStreamSynchronize(stream()));
+    // [r, m] row-major on the host -> [m, r] on the device, through S, a column tile at a time
+    // when S holds no more
+    const int64_t step = nmf->tiled ? nmf->tile_cols : nmf->m;
+    for (int64_t c0 = 0; c0 < nmf->m; c0 += step) {
+      const int64_t len = nmf->m - c0 < step ? nmf->m - c0 : step;
+      DN_HIP(hipMemcpy2D(nmf->S, sizeof(float) * len, H_rm + c0, sizeof(float) * nmf->m,
+                         sizeof(float) * len, (size_t)nmf->r, hipMemcpyHostToDevice));
+      DN_TRY(launch_transpose(nmf->r, len, nmf->S, nmf->H + c0 * nmf->r));
+      DN_HIP(hipStreamSynchronize(stream()));
+    }
   }
+  return 0;
+}
+
+// The matrix may have been planned again for another rank since this handle was made (a second
+// handle, a single-kernel call): make its work lists and workspaces fit this rank again.
+static int products_for(dnpeff_nmf* h) {
+  DN_TRY(csr_ensure_products(h->A, h->r));
+  if (h->tiled) DN_TRY(csr_tile_lists(h->A));
   return 0;
 }
 
@@ -190,6 +323,7 @@ DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
   if (!h->nw_valid) {  // a loss evaluation since the last H update has left A H^T in Nw
+    DN_TRY(products_for(h));
     DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N));
     DN_TRY(launch_spmm_n(A, h->r, h->H));
     DN_TRY(h->prof.end());
@@ -212,14 +346,46 @@ DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   return 0;
 }
 
+// The H update on column tiles: A^T W of a tile into S, then the tile's update written one tile
+// away from the old tile inside Hbuf.  H at the start of Hbuf: the new H goes one tile up and
+// the tiles are walked from the last to the first (a new tile then lands on old tiles that were
+// read already); H one tile up: the new H goes to the start, first tile first.  The tiles are
+// independent of one another, so the order does not change any sum.
+static int update_H_tiled(dnpeff_nmf* h) {
+  dnpeff_csr* A = h->A;
+  const int r = h->r;
+  const int64_t tile = h->tile_cols, n_tiles = ceil_div(h->m, tile);
+  const bool up = h->H == h->Hbuf;
+  float* Hnew = up ? h->Hbuf + tile * r : h->Hbuf;
+  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+  DN_TRY(launch_head_t_product(A, r, h->W));
+  DN_TRY(h->prof.end());
+  for (int64_t q = 0; q < n_tiles; q++) {
+    const int64_t t = up ? n_tiles - 1 - q : q;
+    const int64_t c0 = t * tile, c1 = c0 + tile < h->m ? c0 + tile : h->m;
+    DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+    DN_TRY(launch_spmm_t_tile(A, r, h->W, c0, c1, h->S));
+    DN_TRY(h->prof.end());
+    DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_H));
+    DN_TRY(launch_xg_mu(c1 - c0, r, h->H + c0 * r, h->G, h->S, h->eps, Hnew + c0 * r, nullptr));
+    DN_TRY(h->prof.end());
+  }
+  h->H = Hnew;
+  h->gh_valid = false;
+  return 0;
+}
+
 DN_API int dnpeff_nmf_update_H(dnpeff_nmf* h) {
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
-  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
-  DN_TRY(launch_spmm_t(A, h->r, h->W, h->S));
-  DN_TRY(h->prof.end());
+  DN_TRY(products_for(h));
   DN_TRY(h->prof.begin(DNPEFF_K_GRAM_W));
   DN_TRY(launch_gram(h->n, h->r, h->W, h->G, h->gram_ws));
+  DN_TRY(h->prof.end());
+  h->nw_valid = false;
+  if (h->tiled) return update_H_tiled(h);
+  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+  DN_TRY(launch_spmm_t(A, h->r, h->W, h->S));
   DN_TRY(h->prof.end());
   DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_H));
   if (h->GH && ((uintptr_t)h->H % 16) == 0) {
@@ -231,7 +397,7 @@ DN_API int dnpeff_nmf_update_H(dnpeff_nmf* h) {
   }
   DN_TRY(h->prof.end());
   std::swap(h->H, h->S);
-  h->nw_valid = false;
+  h->Hbuf = h->H;
   return 0;
 }
 
@@ -251,6 +417,7 @@ DN_API int dnpeff_nmf_loss_terms(dnpeff_nmf* h, double* sq_norm_A, double* pos, 
   dnpeff_csr* A = h->A;
   // neg = <W^T A, H> = <A H^T, W>
   if (!h->nw_valid) {
+    DN_TRY(products_for(h));
     DN_TRY(launch_spmm_n(A, h->r, h->H));
     DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
     h->nw_valid = true;
@@ -293,9 +460,16 @@ DN_API int dnpeff_nmf_get_W(dnpeff_nmf* nmf, float* W_nr) {
 DN_API int dnpeff_nmf_get_H(dnpeff_nmf* nmf, float* H_rm) {
   clear_error();
   DN_CHECK(nmf && H_rm, "NULL argument");
-  DN_TRY(launch_transpose(nmf->m, nmf->r, nmf->H, nmf->S));
-  DN_HIP(hipStreamSynchronize(stream()));
-  DN_HIP(hipMemcpy(H_rm, nmf->S, sizeof(float) * nmf->m * nmf->r, hipMemcpyDeviceToHost));
+  // [m, r] on the device -> [r, m] row-major on the host, through S: all at once, or a column
+  // tile at a time when S holds no more (the tiled H update)
+  const int64_t step = nmf->tiled ? nmf->tile_cols : nmf->m;
+  for (int64_t c0 = 0; c0 < nmf->m; c0 += step) {
+    const int64_t len = nmf->m - c0 < step ? nmf->m - c0 : step;
+    DN_TRY(launch_transpose(len, nmf->r, nmf->H + c0 * nmf->r, nmf->S));
+    DN_HIP(hipStreamSynchronize(stream()));
+    DN_HIP(hipMemcpy2D(H_rm + c0, sizeof(float) * nmf->m, nmf->S, sizeof(float) * len,
+                       sizeof(float) * len, (size_t)nmf->r, hipMemcpyDeviceToHost));
+  }
   return 0;
 }
 

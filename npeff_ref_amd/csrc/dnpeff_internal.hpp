@@ -5,6 +5,7 @@
 
 #include <cstdint>
 #include <cstdio>
+#include <vector>
 
 #include "../../include/dnpeff.h"
 
@@ -69,6 +70,31 @@ inline void dfree(void* p) {
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// A device buffer that is freed when it goes out of scope, for temporaries of functions with
+// several exits; release() hands the pointer over to a longer-lived owner.
+template <class T>
+struct dbuf {
+  T* p = nullptr;
+  dbuf() = default;
+  dbuf(const dbuf&) = delete;
+  dbuf& operator=(const dbuf&) = delete;
+  ~dbuf() { dfree(p); }
+  int alloc(int64_t count) {
+    dfree(p);
+    return dmalloc(&p, count);
+  }
+  void reset() {
+    dfree(p);
+    p = nullptr;
+  }
+  T* release() {
+    T* q = p;
+    p = nullptr;
+    return q;
+  }
+  operator T*() const { return p; }
+};
+
 // ---- scans (loader.hip) ----
 // out[i] = sum_{i' < i} (count[i'] >= min_count), i in [0, n]; out has n+1 entries.
 int scan_keep_mask(const int* count, int min_count, int64_t n, int32_t* out);
@@ -115,12 +141,31 @@ int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials);
 int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr);
 
+// Switches for experiments and for tests that force a code path.  Each has an environment
+// variable DNPEFF_<NAME IN CAPITALS> that is read once, when the library is first used, and can be
+// set afterwards with dnpeff_tuning_set(); plans (panels, head, tiles) take their values when they
+// are made, launch paths read no environment.
+struct tuning_t {
+  double dense_fill = 1.0 / 16.0;  // columns held by this fraction of the rows form the dense head (0 = none)
+  double panels = -1.0;            // coarse column panels of A H^T (-1 = by the size of the factor, 0 = none)
+  double sweep_bytes = 3.0 * 1024 * 1024;  // bytes of the factor per swept piece (0 = no swept pieces)
+  double sweep_min = -1.0;         // entries a row must hold per piece on average (-1 = default rule)
+  double sweep_waves = 0.0;        // waves per workgroup of the sweep kernel (0 = as many as fit)
+  double sweep_lag = 0.0;          // pieces the workgroups of an XCD may be apart
+  double sweep_spin = 400.0;       // polls before a workgroup of the sweep stops waiting
+  double spmm_t_slices = 1.0;      // component slices of A^T W
+  double split_bf16 = 1.0;         // matrix products on the bf16 cores with split fp32 operands (0 = fp32 cores)
+  double fused_gram = 1.0;         // rank 128: the H update also produces H^T H
+  double h_tile_mb = 128.0;        // size of a column tile of the tiled H update, MiB of the factor
+  double tiled_h = -1.0;           // tiled H update: 1 = always, 0 = never, -1 = when the full-size buffer does not fit
+  double topk_fast_cap = -1.0;     // top-k: candidate list length that ends the histogram passes (-1 = default)
+  double verbose = 0.0;
+};
+tuning_t& tuning();
+
 // Products of the large matrix-core kernels run on the bf16 matrix cores with every fp32 operand
-// split in three (split_bf16.hpp) unless DNPEFF_SPLIT_BF16=0 selects the fp32 matrix cores.
-inline bool use_split_bf16() {
-  const char* e = getenv("DNPEFF_SPLIT_BF16");
-  return e ? atoi(e) != 0 : true;
-}
+// split in three (split_bf16.hpp) unless the split_bf16 switch selects the fp32 matrix cores.
+inline bool use_split_bf16() { return tuning().split_bf16 != 0.0; }
 
 // Columns present in many rows, held as a dense block in both orientations (head.hip).
 struct dense_head {
@@ -188,6 +233,9 @@ struct dnpeff_csr {
   // (same shape, owned), which carries the derived structures the products use
   dn::dense_head head;
   dnpeff_csr* tail = nullptr;
+  // host copies of head.cols and long_cols (ascending), made when a product runs on column tiles
+  std::vector<int32_t> h_head_cols, h_long_cols;
+  bool h_lists_valid = false;
 };
 
 namespace dn {
@@ -212,4 +260,30 @@ int head_ensure_workspace(dnpeff_csr* A, int r);
 int launch_head_n(const dnpeff_csr* A, int r, const float* H_mr);
 int launch_head_n_add(const dnpeff_csr* A, int r, float* N_nr);
 int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
+// The same in two steps for a result that is produced in column tiles: the product into the head's
+// workspace once, then the rows of the head slots [k0, k1) to T_tile[cols[k] - col0].
+int launch_head_t_product(const dnpeff_csr* A, int r, const float* W_nr);
+int launch_head_t_scatter(const dnpeff_csr* A, int r, int64_t k0, int64_t k1, int64_t col0,
+                          float* T_tile);
+// Rows [col0, col1) of A^T W into T_tile (row j - col0), sparse part and dense head; the head's
+// product must have been launched (launch_head_t_product) and csr_tile_lists(A) built.
+int launch_spmm_t_tile(const dnpeff_csr* A, int r, const float* W_nr, int64_t col0, int64_t col1,
+                       float* T_tile);
+int csr_tile_lists(dnpeff_csr* A);
+// True while the arrays of the row-major copy that the loader calls and dnpeff_csr_download use
+// are there (dnpeff_csr_release or a consuming dnpeff_nmf_create_ex frees them).
+inline bool has_row_major(const dnpeff_csr* A) {
+  return A->rowptr != nullptr && (A->nnz == 0 || (A->colind != nullptr && A->vals != nullptr));
+}
+struct head_choice {
+  int64_t thr = 0;   // columns with at least thr entries form the head (0 = no head)
+  int64_t n_d = 0;
+  double footprint = 0.0;  // bytes of the dense blocks + both sparse copies of the rest
+  bool fits = true;        // footprint within the budget given
+};
+constexpr double NO_BUDGET = 1e300;
+int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, head_choice* out);
+int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense);
+// Frees every array of A that the products A H^T and A^T W do not read.
+int csr_consume_for_products(dnpeff_csr* A);
 }  // namespace dn

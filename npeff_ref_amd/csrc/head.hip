@@ -454,14 +454,15 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// T[cols[k]] = sum over slices of ws[s][k]
+// T[cols[k] - col0] = sum over slices of ws[s][k], k0 <= k < k1
 __global__ void __launch_bounds__(256)
-    k_head_scatter(const float* __restrict__ ws, int64_t slices, int64_t n_d, int64_t n_d_pad, int r,
-                   const int32_t* __restrict__ cols, float* __restrict__ T) {
+    k_head_scatter(const float* __restrict__ ws, int64_t slices, int64_t k0, int64_t k1,
+                   int64_t n_d_pad, int r, const int32_t* __restrict__ cols, int64_t col0,
+                   float* __restrict__ T) {
   const int r4 = r >> 2;
-  const int64_t total = n_d * r4, stride = (int64_t)gridDim.x * 256;
+  const int64_t total = (k1 - k0) * r4, stride = (int64_t)gridDim.x * 256;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
-    const int64_t k = e / r4;
+    const int64_t k = k0 + e / r4;
     const int c = (int)(e % r4);
     float4 out;
     if (slices == 1) {
@@ -474,7 +475,7 @@ __global__ void __launch_bounds__(256)
       }
       out = make_float4((float)s0, (float)s1, (float)s2, (float)s3);
     }
-    reinterpret_cast<float4*>(T + (int64_t)cols[k] * r)[c] = out;
+    reinterpret_cast<float4*>(T + ((int64_t)cols[k] - col0) * r)[c] = out;
   }
 }
 
@@ -546,12 +547,11 @@ int launch_head_n_add(const dnpeff_csr* A, int r, float* N_nr) {
   return 0;
 }
 
-// rows of the head of A^T W (overwrites what the sparse kernels stored there)
-int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
+// slice partials of D^T W into the workspace
+int launch_head_t_product(const dnpeff_csr* A, int r, const float* W_nr) {
   const dense_head& h = A->head;
   if (h.n_d == 0) return 0;
-  DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)W_nr % 16) == 0 && ((uintptr_t)T_mr % 16) == 0,
-           "dense head: workspace or alignment");
+  DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)W_nr % 16) == 0, "dense head: workspace or alignment");
   float* part = h.ws + head_gather_floats(h, r);
   const int64_t slices = head_slices_t(h, r, A->n_rows);
   if (head_uses_split(r)) {
@@ -559,14 +559,30 @@ int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
     float* Wt = h.ws;
     dim3 tg((unsigned)ceil_div(h.n_pad, 32), (unsigned)ceil_div(r, 32));
     hipLaunchKernelGGL(k_transpose_pad, tg, dim3(256), 0, stream(), W_nr, A->n_rows, r, h.n_pad, Wt);
-    DN_TRY(launch_abt_b16(h.cm, h.n_pad, Wt, h.n_pad, A->n_rows, r, h.n_d, h.n_d_pad, slices, part));
-  } else {
-    DN_TRY(launch_ptq(h.rm, h.n_d_pad, A->n_rows, W_nr, r, h.n_d, h.n_d_pad, slices, part));
+    return launch_abt_b16(h.cm, h.n_pad, Wt, h.n_pad, A->n_rows, r, h.n_d, h.n_d_pad, slices, part);
   }
-  hipLaunchKernelGGL(k_head_scatter, dim3(elem_grid(h.n_d * (r / 4))), dim3(256), 0, stream(), part,
-                     slices, h.n_d, h.n_d_pad, r, h.cols, T_mr);
+  return launch_ptq(h.rm, h.n_d_pad, A->n_rows, W_nr, r, h.n_d, h.n_d_pad, slices, part);
+}
+
+// rows of the head slots [k0, k1) of A^T W from the slice partials, to T_tile[cols[k] - col0]
+// (overwrites what the sparse kernels stored there)
+int launch_head_t_scatter(const dnpeff_csr* A, int r, int64_t k0, int64_t k1, int64_t col0,
+                          float* T_tile) {
+  const dense_head& h = A->head;
+  if (h.n_d == 0 || k1 <= k0) return 0;
+  DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)T_tile % 16) == 0, "dense head: workspace or alignment");
+  DN_CHECK(k0 >= 0 && k1 <= h.n_d, "dense head: slots [%lld, %lld) outside the head", (long long)k0,
+           (long long)k1);
+  const float* part = h.ws + head_gather_floats(h, r);
+  hipLaunchKernelGGL(k_head_scatter, dim3(elem_grid((k1 - k0) * (r / 4))), dim3(256), 0, stream(), part,
+                     head_slices_t(h, r, A->n_rows), k0, k1, h.n_d_pad, r, h.cols, col0, T_tile);
   DN_LAUNCH_CHECK();
   return 0;
+}
+
+int launch_head_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr) {
+  DN_TRY(launch_head_t_product(A, r, W_nr));
+  return launch_head_t_scatter(A, r, 0, A->head.n_d, 0, T_mr);
 }
 
 }  // namespace dn

@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstdlib>
 
+#include <cctype>
 #include <cstdarg>
 #include <cstring>
 #include <vector>
@@ -45,6 +46,37 @@ int n_cus() {
     if (g_n_cus <= 0) g_n_cus = 256;
   }
   return g_n_cus;
+}
+
+struct tuning_entry {
+  const char* name;
+  double tuning_t::*field;
+};
+static const tuning_entry g_tuning_table[] = {
+    {"dense_fill", &tuning_t::dense_fill},       {"panels", &tuning_t::panels},
+    {"sweep_bytes", &tuning_t::sweep_bytes},     {"sweep_min", &tuning_t::sweep_min},
+    {"sweep_waves", &tuning_t::sweep_waves},     {"sweep_lag", &tuning_t::sweep_lag},
+    {"sweep_spin", &tuning_t::sweep_spin},       {"spmm_t_slices", &tuning_t::spmm_t_slices},
+    {"split_bf16", &tuning_t::split_bf16},       {"fused_gram", &tuning_t::fused_gram},
+    {"h_tile_mb", &tuning_t::h_tile_mb},         {"tiled_h", &tuning_t::tiled_h},
+    {"topk_fast_cap", &tuning_t::topk_fast_cap}, {"verbose", &tuning_t::verbose},
+};
+
+static tuning_t tuning_from_env() {
+  tuning_t t;
+  for (const tuning_entry& e : g_tuning_table) {
+    char var[64] = "DNPEFF_";
+    size_t k = strlen(var);
+    for (const char* c = e.name; *c && k + 1 < sizeof(var); c++) var[k++] = (char)toupper((unsigned char)*c);
+    var[k] = 0;
+    if (const char* v = getenv(var)) t.*(e.field) = atof(v);
+  }
+  return t;
+}
+
+tuning_t& tuning() {
+  static tuning_t t = tuning_from_env();
+  return t;
 }
 
 struct KeepMaskF {
@@ -410,11 +442,49 @@ static unsigned grid_for(int64_t n, int64_t cap = 1 << 20) {
   return (unsigned)g;
 }
 
+// sum over the columns with count >= thr of their counts (an integer sum: any order)
+__global__ void __launch_bounds__(256)
+    k_sum_selected(const int* __restrict__ count, int64_t n, int thr, unsigned long long* out) {
+  __shared__ unsigned long long sh[256];
+  unsigned long long s = 0;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const int c = count[i];
+    if (c >= thr) s += (unsigned long long)c;
+  }
+  sh[threadIdx.x] = s;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if (threadIdx.x < off) sh[threadIdx.x] += sh[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0 && sh[0]) atomicAdd(out, sh[0]);
+}
+
+// bad += 1 for every column that holds the same row twice in a row of its list (after the stable
+// transposition the entries of one row of a column are adjacent)
+__global__ void __launch_bounds__(256)
+    k_check_repeats(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
+                    int64_t n_cols, int* __restrict__ bad) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x; j < n_cols; j += stride) {
+    const int64_t p1 = colptr[j + 1];
+    int32_t prev = -1;
+    bool rep = false;
+    for (int64_t p = colptr[j]; p < p1; p++) {
+      const int32_t i = rowind[p];
+      rep = rep || i == prev;
+      prev = i;
+    }
+    if (rep) atomicAdd(bad, 1);
+  }
+}
+
 // Drops entries whose table[col] == -1 and renumbers the rest (in place on A).
 static int apply_column_table(dnpeff_csr* A, const int32_t* table, int64_t new_n_cols) {
   hipStream_t st = stream();
-  int64_t* newpos = nullptr;
-  DN_TRY(dmalloc(&newpos, A->nnz + 1));
+  dbuf<int64_t> newpos;
+  DN_TRY(newpos.alloc(A->nnz + 1));
   DN_TRY(scan_kept_entries(A->colind, table, A->nnz, newpos));
   int64_t new_nnz = 0;
   DN_HIP(hipMemcpy(&new_nnz, newpos + A->nnz, sizeof(int64_t), hipMemcpyDeviceToHost));
@@ -423,24 +493,23 @@ static int apply_column_table(dnpeff_csr* A, const int32_t* table, int64_t new_n
                        table);
     DN_LAUNCH_CHECK();
   } else {
-    int32_t* out_col = nullptr;
-    float* out_val = nullptr;
-    DN_TRY(dmalloc(&out_col, new_nnz));
-    DN_TRY(dmalloc(&out_val, new_nnz));
+    dbuf<int32_t> out_col;
+    dbuf<float> out_val;
+    DN_TRY(out_col.alloc(new_nnz));
+    DN_TRY(out_val.alloc(new_nnz));
     hipLaunchKernelGGL(k_compact_entries, dim3(grid_for(A->nnz)), dim3(256), 0, st, A->colind,
-                       A->vals, A->nnz, table, newpos, out_col, out_val);
+                       A->vals, A->nnz, table, newpos.p, out_col.p, out_val.p);
     hipLaunchKernelGGL(k_remap_rowptr, dim3(grid_for(A->n_rows + 1)), dim3(256), 0, st, A->rowptr,
-                       A->n_rows, newpos);
+                       A->n_rows, newpos.p);
     DN_LAUNCH_CHECK();
     DN_HIP(hipStreamSynchronize(st));
     dfree(A->colind);
     dfree(A->vals);
-    A->colind = out_col;
-    A->vals = out_val;
+    A->colind = out_col.release();
+    A->vals = out_val.release();
     A->nnz = new_nnz;
   }
   DN_HIP(hipStreamSynchronize(st));
-  dfree(newpos);
   A->n_cols = new_n_cols;
   return 0;
 }
@@ -469,6 +538,7 @@ static void drop_panels(dnpeff_csr* A) {
 }
 
 static void drop_derived(dnpeff_csr* A) {
+  A->h_lists_valid = false;
   drop_head(A);
   drop_panels(A);
   dfree(A->colptr); A->colptr = nullptr;
@@ -495,7 +565,7 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
   const int P0 = plan.coarse;
   if (P0 <= 0) return 0;
   DN_CHECK(P0 <= MAX_PANELS, "at most %d column panels", MAX_PANELS);
-  DN_CHECK(S->rowptr && S->colptr, "column panels need both copies of the matrix");
+  DN_CHECK(has_row_major(S) && S->colptr, "column panels need both copies of the matrix");
   hipStream_t st = stream();
   // coarse panels: equal numbers of entries
   std::vector<int32_t> coarse((size_t)P0 + 1);
@@ -566,7 +636,7 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
   S->n_plain = n_plain;
   S->n_swept = n_swept;
   S->plan = plan;
-  if (getenv("DNPEFF_VERBOSE"))
+  if (tuning().verbose != 0.0)
     fprintf(stderr, "dnpeff: %d column panels: %d plain, %d cut into %d swept pieces\n", P0, n_plain,
             P0 - n_plain, n_swept);
   dfree(S->partials); S->partials = nullptr; S->partials_floats = 0;
@@ -575,26 +645,29 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
 
 // Panels pay when the gathered factor [n_cols, r] is far larger than the caches and there are
 // rows enough to share a panel's part of it: one coarse panel per ~48 MB of the factor, 8..512
-// (per ~96 MB, 8..256, at the ranks that have swept pieces), and few enough for the (panel, 4
-// rows) workgroups to fit one launch.  On 10,000 x 65.9M,
+// (per ~96 MB, 8..256, at the ranks that have swept pieces), few enough for the (panel, 4
+// rows) workgroups to fit one launch and for the partial sums (one [n_rows, r] block per plain
+// panel) to stay within 3 GB.  On 10,000 x 65.9M,
 // r = 128 (33.7 GB factor): no panels 29.3 ms, 32: 27.8, 128: 23.9, 256: 21.8, 512: 20.1 ms for
 // the gathers, plus 0.1 to 0.8 ms for the sum over panels; 1024 gains 1.1 ms and loses 0.7.
-// DNPEFF_PANELS overrides the number (0 = none).  Swept pieces hold DNPEFF_SWEEP_BYTES of the
+// The `panels` switch overrides the number (0 = none).  Swept pieces hold `sweep_bytes` of the
 // factor each (default 3 MB of the 4 MB L2 of an XCD; 0 = no sweeps) and are made where a row
-// holds DNPEFF_SWEEP_MIN entries per piece on average (default 4, more when there are few rows).
+// holds `sweep_min` entries per piece on average (default 4, more when there are few rows).
 static panel_plan panel_policy(const dnpeff_csr* S, int r) {
+  const tuning_t& tn = tuning();
   int64_t P = 0;
   const double bytes = 4.0 * (double)S->n_cols * r;
-  bool sweeps = spmm_n_sweep_supported(r);
-  if (const char* e = getenv("DNPEFF_SWEEP_BYTES")) sweeps = sweeps && atof(e) > 0.0;
+  const bool sweeps = spmm_n_sweep_supported(r) && tn.sweep_bytes > 0.0;
   if (bytes >= 512e6 && S->n_rows >= 64) {
     // with swept pieces for the panels in between, half as many coarse panels do as well for the
     // gathers and halve the sum over the panels (configs[1]: 19.8 -> 19.4 ms for both)
     P = (int64_t)ceil(bytes / (sweeps ? 96e6 : 48e6));
     if (P < 8) P = 8;
     if (P > (sweeps ? 256 : 512)) P = sweeps ? 256 : 512;
+    const int64_t by_partials = (int64_t)(3.0e9 / (4.0 * (double)S->n_rows * r));
+    if (P > by_partials) P = by_partials < 8 ? 8 : by_partials;
   }
-  if (const char* e = getenv("DNPEFF_PANELS")) P = atoi(e);
+  if (tn.panels >= 0.0) P = (int64_t)tn.panels;
   if (P > 512) P = 512;
   const int64_t row_groups = ceil_div(S->n_rows, 4);
   while (P > 1 && P * row_groups >= ((int64_t)1 << 24)) P /= 2;
@@ -602,8 +675,7 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   panel_plan plan;
   plan.coarse = (int)P;
   if (P > 0 && sweeps) {
-    double sweep_bytes = 3.0 * 1024 * 1024;
-    if (const char* e = getenv("DNPEFF_SWEEP_BYTES")) sweep_bytes = atof(e);
+    double sweep_bytes = tn.sweep_bytes;
     if (sweep_bytes > 1e9) sweep_bytes = 1e9;  // (the kernel addresses a piece with 32 bits)
     plan.sweep_cols = (int)(sweep_bytes / (4.0 * r));
     // a piece must also bring work enough for a sweep step (a wait for the other workgroups of
@@ -611,7 +683,7 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
     plan.sweep_min = 4.0;
     if (S->n_rows > 0 && 20000.0 / (double)S->n_rows > plan.sweep_min)
       plan.sweep_min = 20000.0 / (double)S->n_rows;
-    if (const char* e = getenv("DNPEFF_SWEEP_MIN")) plan.sweep_min = atof(e);
+    if (tn.sweep_min >= 0.0) plan.sweep_min = tn.sweep_min;
     if (plan.sweep_cols <= 0) plan.sweep_cols = 0, plan.sweep_min = 0.0;
   }
   return plan;
@@ -623,6 +695,39 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
   DN_TRY(csr_set_panels(S, panel_policy(S, r)));
   DN_TRY(csr_ensure_partials(S, r));
   return head_ensure_workspace(A, r);
+}
+
+int csr_consume_for_products(dnpeff_csr* A) {
+  DN_HIP(hipStreamSynchronize(stream()));
+  dnpeff_csr* S = sparse_part(A);
+  if (A->tail) {  // the products read the dense head and the tail, not the whole matrix
+    dfree(A->colind); A->colind = nullptr;
+    dfree(A->vals); A->vals = nullptr;
+    dfree(A->chunk_base); A->chunk_base = nullptr; A->n_chunks = 0;
+    dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
+  }
+  if (S->n_panels > 0 && S->nnz > 0) {  // A H^T reads the regrouped copy
+    DN_TRY(csr_ensure_chunks(S));  // (sizes the partial sums; needs the row offsets only)
+    dfree(S->colind); S->colind = nullptr;
+    dfree(S->vals); S->vals = nullptr;
+  }
+  return 0;
+}
+
+int csr_tile_lists(dnpeff_csr* A) {
+  if (A->h_lists_valid) return 0;
+  const dnpeff_csr* S = sparse_part(A);
+  A->h_head_cols.assign((size_t)A->head.n_d, 0);
+  A->h_long_cols.assign((size_t)S->n_long, 0);
+  DN_HIP(hipStreamSynchronize(stream()));
+  if (A->head.n_d)
+    DN_HIP(hipMemcpy(A->h_head_cols.data(), A->head.cols, sizeof(int32_t) * A->head.n_d,
+                     hipMemcpyDeviceToHost));
+  if (S->n_long)
+    DN_HIP(hipMemcpy(A->h_long_cols.data(), S->long_cols, sizeof(int32_t) * S->n_long,
+                     hipMemcpyDeviceToHost));
+  A->h_lists_valid = true;
+  return 0;
 }
 
 int csr_ensure_partials(dnpeff_csr* A, int r) {
@@ -675,6 +780,44 @@ DN_API int dnpeff_sync(void) {
 }
 
 DN_API void* dnpeff_stream(void) { return (void*)stream(); }
+
+DN_API int dnpeff_tuning_set(const char* name, double value) {
+  clear_error();
+  DN_CHECK(name != nullptr, "name is NULL");
+  for (const tuning_entry& e : g_tuning_table)
+    if (strcmp(e.name, name) == 0) {
+      tuning().*(e.field) = value;
+      return 0;
+    }
+  DN_CHECK(false, "no tuning switch named '%s'", name);
+  return 0;
+}
+
+DN_API int dnpeff_tuning_get(const char* name, double* value) {
+  clear_error();
+  DN_CHECK(name && value, "NULL argument");
+  for (const tuning_entry& e : g_tuning_table)
+    if (strcmp(e.name, name) == 0) {
+      *value = tuning().*(e.field);
+      return 0;
+    }
+  DN_CHECK(false, "no tuning switch named '%s'", name);
+  return 0;
+}
+
+DN_API int dnpeff_tuning_reset(void) {
+  tuning() = tuning_from_env();
+  return 0;
+}
+
+DN_API int dnpeff_device_memory(int64_t* free_bytes, int64_t* total_bytes) {
+  clear_error();
+  size_t f = 0, t = 0;
+  DN_HIP(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = (int64_t)f;
+  if (total_bytes) *total_bytes = (int64_t)t;
+  return 0;
+}
 
 DN_API int dnpeff_dev_malloc(int64_t bytes, void** out) {
   clear_error();
@@ -809,7 +952,7 @@ DN_API int dnpeff_csr_from_pef(int64_t n_rows, int64_t k, int64_t dense_fisher_s
 
 DN_API int dnpeff_csr_normalize_rows(dnpeff_csr* A, const float* norms_host, float eps) {
   clear_error();
-  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(A && has_row_major(A), "matrix is NULL or its row-major arrays were released");
   DN_CHECK(norms_host != nullptr || A->n_rows == 0, "norms is NULL");
   if (A->n_rows == 0) return 0;
   float* norms = nullptr;
@@ -827,41 +970,39 @@ DN_API int dnpeff_csr_normalize_rows(dnpeff_csr* A, const float* norms_host, flo
 
 DN_API int dnpeff_csr_compact_columns(dnpeff_csr* A, int min_count) {
   clear_error();
-  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(A && has_row_major(A), "matrix is NULL or its row-major arrays were released");
   hipStream_t st = stream();
   drop_derived(A);
   const int64_t m_full = A->n_cols;
-  int* count = nullptr;
-  int32_t *pos = nullptr, *og_to_new = nullptr, *new_to_og = nullptr;
-  DN_TRY(dmalloc(&count, m_full));
+  dbuf<int> count;
+  dbuf<int32_t> pos, og_to_new, new_to_og;
+  DN_TRY(count.alloc(m_full));
   DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m_full > 0 ? m_full : 1), st));
   hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
-                     count);
+                     count.p);
   DN_LAUNCH_CHECK();
-  DN_TRY(dmalloc(&pos, m_full + 1));
+  DN_TRY(pos.alloc(m_full + 1));
   DN_TRY(scan_keep_mask(count, min_count, m_full, pos));
   int32_t m_new = 0;
   DN_HIP(hipMemcpy(&m_new, pos + m_full, sizeof(int32_t), hipMemcpyDeviceToHost));
-  DN_TRY(dmalloc(&og_to_new, m_full));
-  DN_TRY(dmalloc(&new_to_og, (int64_t)m_new));
-  hipLaunchKernelGGL(k_build_maps, dim3(grid_for(m_full)), dim3(256), 0, st, count, min_count, pos,
-                     m_full, og_to_new, new_to_og);
+  DN_TRY(og_to_new.alloc(m_full));
+  DN_TRY(new_to_og.alloc((int64_t)m_new));
+  hipLaunchKernelGGL(k_build_maps, dim3(grid_for(m_full)), dim3(256), 0, st, count.p, min_count,
+                     pos.p, m_full, og_to_new.p, new_to_og.p);
   DN_LAUNCH_CHECK();
   DN_HIP(hipStreamSynchronize(st));
-  dfree(count);
-  dfree(pos);
+  count.reset();
+  pos.reset();
   A->full_dense_size = m_full;
-  int s = apply_column_table(A, og_to_new, (int64_t)m_new);
-  dfree(og_to_new);
-  if (s) { dfree(new_to_og); return s; }
+  DN_TRY(apply_column_table(A, og_to_new, (int64_t)m_new));
   dfree(A->kept);
-  A->kept = new_to_og;
+  A->kept = new_to_og.release();
   return 0;
 }
 
 DN_API int dnpeff_csr_retain_columns(dnpeff_csr* A, const int32_t* kept, int64_t n_kept) {
   clear_error();
-  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(A && has_row_major(A), "matrix is NULL or its row-major arrays were released");
   DN_CHECK(n_kept >= 0 && (kept || n_kept == 0), "kept is NULL");
   for (int64_t i = 0; i < n_kept; i++)
     DN_CHECK(kept[i] >= 0 && kept[i] < A->n_cols, "kept[%lld] = %d outside [0, %lld)",
@@ -901,7 +1042,7 @@ DN_API int dnpeff_csr_full_dense_size(const dnpeff_csr* A, int64_t* out) {
 
 DN_API int dnpeff_csr_download(const dnpeff_csr* A, int64_t* rowptr, int32_t* colind, float* vals) {
   clear_error();
-  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
+  DN_CHECK(A && has_row_major(A), "matrix is NULL or its row-major arrays were released");
   DN_HIP(hipStreamSynchronize(stream()));
   if (rowptr)
     DN_HIP(hipMemcpy(rowptr, A->rowptr, sizeof(int64_t) * (A->n_rows + 1), hipMemcpyDeviceToHost));
@@ -943,89 +1084,168 @@ DN_API int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out) {
   return 0;
 }
 
-DN_API int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* n_dense) {
-  clear_error();
-  DN_CHECK(A && A->rowptr, "matrix is NULL or released");
-  DN_CHECK(min_fill <= 1.0, "min_fill %g above 1", min_fill);
-  hipStream_t st = stream();
-  drop_derived(A);
-  if (n_dense) *n_dense = 0;
-  if (min_fill <= 0.0) return 0;
+// rowptr_out[i] = newpos[rowptr[i]]
+__global__ void __launch_bounds__(256)
+    k_map_rowptr(const int64_t* __restrict__ rowptr, int64_t n_rows, const int64_t* __restrict__ newpos,
+                 int64_t* __restrict__ rowptr_out) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i <= n_rows; i += stride)
+    rowptr_out[i] = newpos[rowptr[i]];
+}
+
+namespace dn {
+
+// Which columns form the dense head.  Candidates are the thresholds thr0, 2 thr0, 4 thr0, ...
+// (thr0 = ceil(min_fill n_rows)) and "no head"; a candidate is admissible when both dense blocks
+// stay below an eighth of the device memory; its footprint is the two blocks plus both sparse
+// copies of the remaining entries (16 bytes each).  The choice is the first admissible candidate
+// whose footprint is within `budget` bytes (NO_BUDGET: the first admissible one), else the
+// admissible candidate with the smallest footprint (fits = false).
+int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, head_choice* out) {
+  *out = head_choice();
+  out->footprint = 16.0 * (double)A->nnz;
+  out->fits = out->footprint <= budget;
   const int64_t m = A->n_cols, n = A->n_rows;
-  if (m == 0 || n == 0 || A->nnz == 0) return 0;
-  int64_t thr = (int64_t)ceil(min_fill * (double)n);
-  if (thr < 1) thr = 1;
-  int* count = nullptr;
-  int32_t *pos = nullptr, *slot_of = nullptr, *cols = nullptr, *table = nullptr;
-  DN_TRY(dmalloc(&count, m));
+  if (min_fill <= 0.0 || m == 0 || n == 0 || A->nnz == 0) return 0;
+  DN_CHECK(has_row_major(A), "matrix is NULL or its row-major arrays were released");
+  hipStream_t st = stream();
+  dbuf<int> count;
+  dbuf<int32_t> pos;
+  dbuf<unsigned long long> zsum;
+  DN_TRY(count.alloc(m));
+  DN_TRY(pos.alloc(m + 1));
+  DN_TRY(zsum.alloc(1));
   DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)m, st));
   hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
-                     count);
+                     count.p);
   DN_LAUNCH_CHECK();
-  DN_TRY(dmalloc(&pos, m + 1));
-  // both dense blocks together stay below an eighth of the device memory: raise the bar
-  // until they do
   size_t free_b = 0, total_b = 0;
   DN_HIP(hipMemGetInfo(&free_b, &total_b));
   const int64_t n_pad = ceil_div(n, 128) * 128;
-  int32_t n_d = 0;
-  for (;;) {
-    DN_CHECK(thr <= (int64_t)INT32_MAX, "dense head: threshold overflow");
+  int64_t thr = (int64_t)ceil(min_fill * (double)n);
+  if (thr < 1) thr = 1;
+  head_choice best = *out;  // "no head"
+  bool have_fit = false;
+  for (; thr <= n && thr <= (int64_t)INT32_MAX; thr *= 2) {
+    int32_t n_d = 0;
+    unsigned long long z_head = 0;
     DN_TRY(scan_keep_mask(count, (int)thr, m, pos));
     DN_HIP(hipMemcpy(&n_d, pos + m, sizeof(int32_t), hipMemcpyDeviceToHost));
-    const double bytes = 2.0 * 4.0 * (double)n_pad * (double)(ceil_div(n_d, 128) * 128);
-    if (bytes <= (double)total_b / 8.0 || thr > n) break;
-    thr *= 2;
+    if (n_d == 0) break;
+    DN_HIP(hipMemsetAsync(zsum, 0, sizeof(unsigned long long), st));
+    hipLaunchKernelGGL(k_sum_selected, dim3(grid_for(m, 4096)), dim3(256), 0, st, count.p, m, (int)thr,
+                       zsum.p);
+    DN_LAUNCH_CHECK();
+    DN_HIP(hipMemcpy(&z_head, zsum, sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    const double blocks = 2.0 * 4.0 * (double)n_pad * (double)(ceil_div(n_d, 128) * 128);
+    if (blocks > (double)total_b / 8.0) continue;
+    head_choice c;
+    c.thr = thr;
+    c.n_d = n_d;
+    c.footprint = blocks + 16.0 * (double)(A->nnz - (int64_t)z_head);
+    c.fits = c.footprint <= budget;
+    if (c.fits) {
+      best = c;
+      have_fit = true;
+      break;
+    }
+    if (c.footprint < best.footprint) best = c;
   }
-  if (n_d == 0 || thr > n) {
-    dfree(count); dfree(pos);
-    return 0;
+  if (!have_fit && out->fits) return 0;  // no head fits the budget, a head does not
+  *out = best;
+  return 0;
+}
+
+// Moves the columns with at least thr entries into the dense head.
+int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense) {
+  hipStream_t st = stream();
+  drop_derived(A);
+  if (n_dense) *n_dense = 0;
+  const int64_t m = A->n_cols, n = A->n_rows;
+  if (thr <= 0 || thr > n || m == 0 || A->nnz == 0) return 0;
+  DN_CHECK(has_row_major(A), "matrix is NULL or its row-major arrays were released");
+  dbuf<int> count;
+  dbuf<int32_t> pos, slot_of, cols, table;
+  DN_TRY(count.alloc(m));
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)m, st));
+  hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
+                     count.p);
+  DN_LAUNCH_CHECK();
+  DN_TRY(pos.alloc(m + 1));
+  DN_TRY(scan_keep_mask(count, (int)thr, m, pos));
+  int32_t n_d = 0;
+  DN_HIP(hipMemcpy(&n_d, pos + m, sizeof(int32_t), hipMemcpyDeviceToHost));
+  if (n_d == 0) return 0;
+  const int64_t n_pad = ceil_div(n, 128) * 128, n_d_pad = ceil_div(n_d, 128) * 128;
+  DN_TRY(slot_of.alloc(m));
+  DN_TRY(cols.alloc((int64_t)n_d));
+  DN_TRY(table.alloc(m));
+  hipLaunchKernelGGL(k_build_maps, dim3(grid_for(m)), dim3(256), 0, st, count.p, (int)thr, pos.p, m,
+                     slot_of.p, cols.p);
+  hipLaunchKernelGGL(k_tail_table, dim3(grid_for(m)), dim3(256), 0, st, slot_of.p, m, table.p);
+  DN_LAUNCH_CHECK();
+  DN_HIP(hipStreamSynchronize(st));
+  count.reset();
+  pos.reset();
+  dbuf<float> cm, rm;
+  DN_TRY(cm.alloc(n_d_pad * n_pad));
+  DN_TRY(rm.alloc(n_pad * n_d_pad));
+  DN_HIP(hipMemsetAsync(cm, 0, sizeof(float) * (size_t)(n_d_pad * n_pad), st));
+  DN_HIP(hipMemsetAsync(rm, 0, sizeof(float) * (size_t)(n_pad * n_d_pad), st));
+  hipLaunchKernelGGL(k_head_fill, dim3(grid_for(n * 256)), dim3(256), 0, st, A->rowptr, A->colind,
+                     A->vals, n, slot_of.p, cm.p, n_pad, rm.p, n_d_pad);
+  DN_LAUNCH_CHECK();
+  // the remaining entries: the row-major arrays without the head's columns, written straight
+  // into the tail's own arrays (positions from a scan over the entries)
+  dnpeff_csr* T = new dnpeff_csr();
+  T->n_rows = n; T->n_cols = m; T->full_dense_size = A->full_dense_size;
+  int status = 0;
+  {
+    dbuf<int64_t> newpos;
+    status = newpos.alloc(A->nnz + 1) || scan_kept_entries(A->colind, table, A->nnz, newpos);
+    if (!status && hipMemcpy(&T->nnz, newpos + A->nnz, sizeof(int64_t), hipMemcpyDeviceToHost) != hipSuccess) {
+      set_error("dense head: reading the size of the sparse part failed");
+      status = 1;
+    }
+    if (!status)
+      status = dmalloc(&T->rowptr, n + 1) || dmalloc(&T->colind, T->nnz) || dmalloc(&T->vals, T->nnz);
+    if (!status) {
+      hipLaunchKernelGGL(k_compact_entries, dim3(grid_for(A->nnz)), dim3(256), 0, st, A->colind,
+                         A->vals, A->nnz, table.p, newpos.p, T->colind, T->vals);
+      hipLaunchKernelGGL(k_map_rowptr, dim3(grid_for(n + 1)), dim3(256), 0, st, A->rowptr, n, newpos.p,
+                         T->rowptr);
+      if (hipGetLastError() != hipSuccess || hipStreamSynchronize(st) != hipSuccess) {
+        set_error("dense head: building the sparse part failed");
+        status = 1;
+      }
+    }
   }
-  const int64_t n_d_pad = ceil_div(n_d, 128) * 128;
-  int s = dmalloc(&slot_of, m) || dmalloc(&cols, (int64_t)n_d) || dmalloc(&table, m);
-  if (!s) {
-    hipLaunchKernelGGL(k_build_maps, dim3(grid_for(m)), dim3(256), 0, st, count, (int)thr, pos, m,
-                       slot_of, cols);
-    hipLaunchKernelGGL(k_tail_table, dim3(grid_for(m)), dim3(256), 0, st, slot_of, m, table);
+  if (status) {
+    dnpeff_csr_destroy(T);
+    return status;
   }
   dense_head& h = A->head;
-  if (!s) s = dmalloc(&h.cm, n_d_pad * n_pad) || dmalloc(&h.rm, n_pad * n_d_pad);
-  if (!s && (hipMemsetAsync(h.cm, 0, sizeof(float) * (size_t)(n_d_pad * n_pad), st) != hipSuccess ||
-             hipMemsetAsync(h.rm, 0, sizeof(float) * (size_t)(n_pad * n_d_pad), st) != hipSuccess)) {
-    set_error("dense head: clearing the blocks failed");
-    s = 1;
-  }
-  if (!s) {
-    hipLaunchKernelGGL(k_head_fill, dim3(grid_for(n * 256)), dim3(256), 0, st, A->rowptr, A->colind,
-                       A->vals, n, slot_of, h.cm, n_pad, h.rm, n_d_pad);
-    if (hipGetLastError() != hipSuccess) { set_error("dense head: launch failed"); s = 1; }
-  }
-  // the remaining entries: a copy of the row-major arrays without the head's columns
-  dnpeff_csr* T = nullptr;
-  if (!s) {
-    T = new dnpeff_csr();
-    T->n_rows = n; T->n_cols = m; T->nnz = A->nnz; T->full_dense_size = A->full_dense_size;
-    s = dmalloc(&T->rowptr, n + 1) || dmalloc(&T->colind, A->nnz) || dmalloc(&T->vals, A->nnz);
-    if (!s && (hipMemcpyAsync(T->rowptr, A->rowptr, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToDevice, st) != hipSuccess ||
-               hipMemcpyAsync(T->colind, A->colind, sizeof(int32_t) * A->nnz, hipMemcpyDeviceToDevice, st) != hipSuccess ||
-               hipMemcpyAsync(T->vals, A->vals, sizeof(float) * A->nnz, hipMemcpyDeviceToDevice, st) != hipSuccess)) {
-      set_error("dense head: copying the entries failed");
-      s = 1;
-    }
-    if (!s) s = apply_column_table(T, table, m);
-  }
-  (void)hipStreamSynchronize(st);
-  dfree(count); dfree(pos); dfree(slot_of); dfree(table);
-  if (s) {
-    if (T) dnpeff_csr_destroy(T);
-    dfree(cols);
-    drop_head(A);
-    return s;
-  }
-  h.n_d = n_d; h.n_d_pad = n_d_pad; h.n_pad = n_pad; h.cols = cols;
+  h.n_d = n_d; h.n_d_pad = n_d_pad; h.n_pad = n_pad;
+  h.cols = cols.release(); h.cm = cm.release(); h.rm = rm.release();
   A->tail = T;
   if (n_dense) *n_dense = n_d;
   return 0;
+}
+
+}  // namespace dn
+
+DN_API int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* n_dense) {
+  clear_error();
+  DN_CHECK(A && has_row_major(A), "matrix is NULL or its row-major arrays were released");
+  DN_CHECK(min_fill <= 1.0, "min_fill %g above 1", min_fill);
+  if (n_dense) *n_dense = 0;
+  if (min_fill <= 0.0) {
+    drop_derived(A);
+    return 0;
+  }
+  head_choice c;
+  DN_TRY(choose_dense_head(A, min_fill, NO_BUDGET, &c));
+  return split_dense_head_at(A, c.thr, n_dense);
 }
 
 DN_API int dnpeff_op_threshold_compact(int64_t count, const float* x, float divisor, float threshold,
@@ -1065,20 +1285,23 @@ DN_API int dnpeff_csr_build_transpose(dnpeff_csr* A) {
   clear_error();
   DN_CHECK(A != nullptr, "matrix is NULL");
   if (A->colptr) return 0;
-  DN_CHECK(A->rowptr != nullptr, "row-major copy of the matrix was released");
+  DN_CHECK(has_row_major(A), "row-major copy of the matrix was released");
   hipStream_t st = stream();
   const int64_t m = A->n_cols;
-  int* count = nullptr;
-  DN_TRY(dmalloc(&count, m));
-  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m > 0 ? m : 1), st));
+  dbuf<int> count;
+  dbuf<int64_t> colptr;
+  dbuf<int32_t> rowind, pos, long_cols;
+  dbuf<float> tvals;
+  DN_TRY(count.alloc(m + 1));  // (the last element counts columns with a repeated row)
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m + 1), st));
   hipLaunchKernelGGL(k_col_hist, dim3(grid_for(A->nnz, 65536)), dim3(256), 0, st, A->colind, A->nnz,
-                     count);
+                     count.p);
   DN_LAUNCH_CHECK();
-  DN_TRY(dmalloc(&A->colptr, m + 1));
-  DN_TRY(scan_counts_i64(count, m, A->colptr));
-  DN_TRY(dmalloc(&A->rowind, A->nnz));
-  DN_TRY(dmalloc(&A->tvals, A->nnz));
-  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m > 0 ? m : 1), st));
+  DN_TRY(colptr.alloc(m + 1));
+  DN_TRY(scan_counts_i64(count, m, colptr));
+  DN_TRY(rowind.alloc(A->nnz));
+  DN_TRY(tvals.alloc(A->nnz));
+  DN_HIP(hipMemsetAsync(count, 0, sizeof(int) * (size_t)(m + 1), st));
   std::vector<int64_t> rowptr((size_t)A->n_rows + 1);
   DN_HIP(hipMemcpy(rowptr.data(), A->rowptr, sizeof(int64_t) * (A->n_rows + 1),
                    hipMemcpyDeviceToHost));
@@ -1086,27 +1309,41 @@ DN_API int dnpeff_csr_build_transpose(dnpeff_csr* A) {
     int64_t len = rowptr[i + 1] - rowptr[i];
     if (len <= 0) continue;
     hipLaunchKernelGGL(k_transpose_row, dim3((unsigned)ceil_div(len, 256)), dim3(256), 0, st,
-                       (int32_t)i, rowptr[i], rowptr[i + 1], A->colind, A->vals, A->colptr, count,
-                       A->rowind, A->tvals);
+                       (int32_t)i, rowptr[i], rowptr[i + 1], A->colind, A->vals, colptr.p, count.p,
+                       rowind.p, tvals.p);
   }
   DN_LAUNCH_CHECK();
-  DN_HIP(hipStreamSynchronize(st));
-  dfree(count);
+  // A row that holds a column twice puts two entries of that row next to each other in the
+  // column's list, in an order that the hardware decides: such a matrix has no deterministic
+  // transposed copy (nor is it a valid PEF matrix: top-k indices are distinct) and is refused.
+  hipLaunchKernelGGL(k_check_repeats, dim3(grid_for(m, 65536)), dim3(256), 0, st, colptr.p, rowind.p, m,
+                     count.p + m);
+  DN_LAUNCH_CHECK();
+  int repeats = 0;
+  DN_HIP(hipMemcpy(&repeats, count.p + m, sizeof(int), hipMemcpyDeviceToHost));
+  DN_CHECK(repeats == 0,
+           "%d column(s) hold the same row more than once: duplicate (row, column) entries are not "
+           "supported by the products",
+           repeats);
+  count.reset();
   // list of long columns for A^T W
-  int32_t* pos = nullptr;
-  DN_TRY(dmalloc(&pos, m + 1));
-  DN_TRY(scan_long_cols(A->colptr, SPMM_T_LONG, m, pos));
+  DN_TRY(pos.alloc(m + 1));
+  DN_TRY(scan_long_cols(colptr, SPMM_T_LONG, m, pos));
   int32_t n_long = 0;
   DN_HIP(hipMemcpy(&n_long, pos + m, sizeof(int32_t), hipMemcpyDeviceToHost));
-  A->n_long = n_long;
-  DN_TRY(dmalloc(&A->long_cols, (int64_t)n_long));
+  DN_TRY(long_cols.alloc((int64_t)n_long));
   if (n_long) {
-    hipLaunchKernelGGL(k_collect_long, dim3(grid_for(m)), dim3(256), 0, st, A->colptr, SPMM_T_LONG,
-                       m, pos, A->long_cols);
+    hipLaunchKernelGGL(k_collect_long, dim3(grid_for(m)), dim3(256), 0, st, colptr.p, SPMM_T_LONG, m,
+                       pos.p, long_cols.p);
     DN_LAUNCH_CHECK();
   }
   DN_HIP(hipStreamSynchronize(st));
-  dfree(pos);
+  A->colptr = colptr.release();
+  A->rowind = rowind.release();
+  A->tvals = tvals.release();
+  A->long_cols = long_cols.release();
+  A->n_long = n_long;
+  A->h_lists_valid = false;
   return 0;
 }
 

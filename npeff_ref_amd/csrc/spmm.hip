@@ -10,6 +10,7 @@
 // reproducible run to run.
 #include "dnpeff_internal.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 #include <utility>
@@ -782,7 +783,8 @@ template <class GT>
 __global__ void __launch_bounds__(256)
     k_spmm_t_long(const int32_t* __restrict__ long_cols, const int64_t* __restrict__ colptr,
                   const int32_t* __restrict__ rowind, const float* __restrict__ tvals, int r,
-                  int n_slices, const float* __restrict__ W, float* __restrict__ T, bool w_small) {
+                  int n_slices, const float* __restrict__ W, float* __restrict__ T, bool w_small,
+                  int64_t col0) {
   extern __shared__ __align__(16) float red_dyn[];  // [4][width]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int slice = blockIdx.x % n_slices, width = r / n_slices;
@@ -803,7 +805,7 @@ __global__ void __launch_bounds__(256)
     s += red_dyn[width + c];
     s += red_dyn[2 * width + c];
     s += red_dyn[3 * width + c];
-    T[j * r + slice * width + c] = s;
+    T[(j - col0) * r + slice * width + c] = s;  // (T starts at column col0)
   }
 }
 
@@ -963,8 +965,7 @@ static sweep_shape sweep_shape_for(int64_t n_rows, int r, int max_waves) {
   sweep_shape best{};
   const int64_t wgs = (int64_t)n_cus() * 2 / SWEEP_XCDS * SWEEP_XCDS;
   const int rows_cap = SWEEP_LDS_BYTES / (4 * r);
-  int forced = 0;
-  if (const char* e = getenv("DNPEFF_SWEEP_WAVES")) forced = atoi(e);
+  int forced = (int)tuning().sweep_waves;
   if (forced < 1 || forced > max_waves) forced = 0;
   for (int waves = max_waves; waves >= 2; waves -= 2) {
     const int w = forced ? forced : waves;
@@ -1018,7 +1019,7 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
   const sweep_shape sh = sweep_shape_for(A->n_rows, r, max_waves);
   DN_CHECK(sh.waves > 0, "no sweep shape for rank %d", r);
   static bool told = false;
-  if (!told && getenv("DNPEFF_VERBOSE")) {
+  if (!told && tuning().verbose != 0.0) {
     told = true;
     fprintf(stderr,
             "dnpeff: sweep kernel with %d registers: %lld workgroups of %d waves, %d rows each, "
@@ -1027,9 +1028,7 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
             (long long)sh.rows_per_pass);
   }
   const int32_t* swept = A->panel_ids + A->n_plain;
-  int lag = 0, spin_max = 400;
-  if (const char* e = getenv("DNPEFF_SWEEP_LAG")) lag = atoi(e);
-  if (const char* e = getenv("DNPEFF_SWEEP_SPIN")) spin_max = atoi(e);
+  int lag = (int)tuning().sweep_lag, spin_max = (int)tuning().sweep_spin;
   if (lag < 0) lag = 0;
   const size_t lds = sizeof(float) * (size_t)sh.rows_wg * r;
   for (int64_t pass = 0; pass < sh.n_pass; pass++) {
@@ -1111,45 +1110,46 @@ int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float
 
 // Component slices for A^T W.  Measured on configs[1] (n = 10,000, r = 128): 1 slice 29 ms,
 // 2 slices 37 ms, 4 slices 64 ms -- re-reading the entries once per slice costs more than the
-// better L2 residency of W gains, so the default is 1.  DNPEFF_SPMM_T_SLICES = 2, 4 or 8
+// better L2 residency of W gains, so the default is 1.  The spmm_t_slices switch (2, 4 or 8)
 // selects a sliced launch (for experiments on other shapes).
 static int spmm_t_slices(int64_t /*n*/, int r) {
-  if (const char* e = getenv("DNPEFF_SPMM_T_SLICES")) {
-    int v = atoi(e);
-    if ((v == 1 || v == 2 || v == 4 || v == 8) && r % v == 0 && (r / v) % 4 == 0) return v;
-  }
+  const int v = (int)tuning().spmm_t_slices;
+  if ((v == 2 || v == 4 || v == 8) && r % v == 0 && (r / v) % 4 == 0) return v;
   return 1;
 }
 
-int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_mr) {
-  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
-  const dnpeff_csr* A = sparse_part(A_full);
+// The sparse part of rows [col0, col1) of A^T W into T (row j - col0); long_cols[l0 .. l1) are the
+// long columns in that range.
+static int launch_spmm_t_sparse(const dnpeff_csr* A, int r, const float* W_nr, float* T, int64_t col0,
+                                int64_t col1, int64_t l0, int64_t l1) {
   DN_CHECK(A->colptr != nullptr, "matrix has no transposed copy");
-  if (A->n_cols == 0) return 0;
-  const bool aligned = ((uintptr_t)T_mr % 16) == 0 && ((uintptr_t)W_nr % 16) == 0;
+  const int64_t m = col1 - col0;
+  if (m <= 0) return 0;
+  const int64_t* colptr = A->colptr + col0;
+  const bool aligned = ((uintptr_t)T % 16) == 0 && ((uintptr_t)W_nr % 16) == 0;
   const int n_slices = (aligned && r % 4 == 0) ? spmm_t_slices(A->n_rows, r) : 1;
   const int width = r / n_slices;
   // one wave per (column, slice); a launch holds at most 2^32 threads, so beyond 2^23 workgroups
   // each one loops over several column groups
-  int64_t wgs = ceil_div(A->n_cols, 4) * n_slices;
+  int64_t wgs = ceil_div(m, 4) * n_slices;
   const int64_t max_wgs = ((int64_t)1 << 23) / n_slices * n_slices;
   if (wgs > max_wgs) wgs = max_wgs;
   dim3 grid((unsigned)wgs), block(256);
   const bool grouped = aligned && r % 4 == 0 && n_slices == 1;
   const bool w_small = (double)A->n_rows * r * 4.0 < 4.0e9;  // 32-bit offsets into W
   if (grouped) {
-    dim3 gg((unsigned)ceil_div(A->n_cols, 4 * SPMM_T_COLS));
+    dim3 gg((unsigned)ceil_div(m, 4 * SPMM_T_COLS));
     const int r4 = r / 4;
-#define DN_GROUPED2(LPR, T, FULL, SMALL)                                                       \
-  hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T, FULL, SMALL>), gg, block, 0, stream(), A->colptr, \
-                     A->rowind, A->tvals, A->n_cols, r, W_nr, T_mr)
-#define DN_GROUPED(LPR, T)                                     \
-  do {                                                         \
-    const bool full = r == 4 * LPR * T;                        \
-    if (full && w_small24) DN_GROUPED2(LPR, T, true, true);    \
-    else if (full) DN_GROUPED2(LPR, T, true, false);           \
-    else if (w_small24) DN_GROUPED2(LPR, T, false, true);      \
-    else DN_GROUPED2(LPR, T, false, false);                    \
+#define DN_GROUPED2(LPR, T_, FULL, SMALL)                                                     \
+  hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T_, FULL, SMALL>), gg, block, 0, stream(), colptr, \
+                     A->rowind, A->tvals, m, r, W_nr, T)
+#define DN_GROUPED(LPR, T_)                                     \
+  do {                                                          \
+    const bool full = r == 4 * LPR * T_;                        \
+    if (full && w_small24) DN_GROUPED2(LPR, T_, true, true);    \
+    else if (full) DN_GROUPED2(LPR, T_, true, false);           \
+    else if (w_small24) DN_GROUPED2(LPR, T_, false, true);      \
+    else DN_GROUPED2(LPR, T_, false, false);                    \
   } while (0)
     const bool w_small24 = w_small && A->n_rows < ((int64_t)1 << 24);
     if (r4 <= 4) DN_GROUPED(4, 1);
@@ -1165,20 +1165,44 @@ int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_m
   dispatch_gather(width, aligned, [&](auto tag) {
     using GT = typename decltype(tag)::type;
     if (!grouped)
-      hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), A->colptr, A->rowind,
-                         A->tvals, A->n_cols, r, n_slices, W_nr, T_mr, w_small);
-    if (A->n_long > 0) {
-      dim3 grid_l((unsigned)(A->n_long * n_slices));
+      hipLaunchKernelGGL((k_spmm_t_short<GT>), grid, block, 0, stream(), colptr, A->rowind, A->tvals,
+                         m, r, n_slices, W_nr, T, w_small);
+    if (l1 > l0) {
+      dim3 grid_l((unsigned)((l1 - l0) * n_slices));
       const size_t lds = sizeof(float) * 4 * (size_t)width;
-      hipLaunchKernelGGL((k_spmm_t_long<GT>), grid_l, block, lds, stream(), A->long_cols,
-                         A->colptr, A->rowind, A->tvals, r, n_slices, W_nr, T_mr, w_small);
+      hipLaunchKernelGGL((k_spmm_t_long<GT>), grid_l, block, lds, stream(), A->long_cols + l0,
+                         A->colptr, A->rowind, A->tvals, r, n_slices, W_nr, T, w_small, col0);
     }
     return 0;
   });
   DN_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_spmm_t(const dnpeff_csr* A_full, int r, const float* W_nr, float* T_mr) {
+  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
+  const dnpeff_csr* A = sparse_part(A_full);
+  DN_TRY(launch_spmm_t_sparse(A, r, W_nr, T_mr, 0, A->n_cols, 0, A->n_long));
   // the head's rows of the result were stored as zeros above (its columns are empty in the
   // sparse part); the dense product overwrites them
   return launch_head_t(A_full, r, W_nr, T_mr);
+}
+
+int launch_spmm_t_tile(const dnpeff_csr* A_full, int r, const float* W_nr, int64_t col0,
+                       int64_t col1, float* T_tile) {
+  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
+  DN_CHECK(A_full->h_lists_valid, "matrix has no host lists for column tiles");
+  const dnpeff_csr* A = sparse_part(A_full);
+  DN_CHECK(0 <= col0 && col0 <= col1 && col1 <= A->n_cols, "column tile [%lld, %lld) outside the matrix",
+           (long long)col0, (long long)col1);
+  const std::vector<int32_t>& lc = A_full->h_long_cols;
+  const int64_t l0 = std::lower_bound(lc.begin(), lc.end(), (int32_t)col0) - lc.begin();
+  const int64_t l1 = std::lower_bound(lc.begin(), lc.end(), (int32_t)col1) - lc.begin();
+  DN_TRY(launch_spmm_t_sparse(A, r, W_nr, T_tile, col0, col1, l0, l1));
+  const std::vector<int32_t>& hc = A_full->h_head_cols;
+  const int64_t k0 = std::lower_bound(hc.begin(), hc.end(), (int32_t)col0) - hc.begin();
+  const int64_t k1 = std::lower_bound(hc.begin(), hc.end(), (int32_t)col1) - hc.begin();
+  return launch_head_t_scatter(A_full, r, k0, k1, col0, T_tile);
 }
 
 int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials) {

@@ -366,7 +366,7 @@ DN_API int dnpeff_topk_rows(int64_t n_rows, int64_t count, int64_t k, const floa
     return most;
   };
   int64_t kp = 1, cap = TOPK_FAST_CAP;
-  if (const char* e = getenv("DNPEFF_TOPK_FAST_CAP")) cap = atoll(e);  // tests: force the deeper paths
+  if (tuning().topk_fast_cap >= 0.0) cap = (int64_t)tuning().topk_fast_cap;  // tests: force the deeper paths
   // while the k-th entry's bin is crowded, decide the next bits of the key (one more read each)
   const int shifts[2] = {10, 0}, bits[2] = {11, 10};
   int64_t most = longest_list();

@@ -31,6 +31,16 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture
+def tune():
+    """tune(name, value) sets a switch of the library (dnpeff_tuning_set) for the test; all
+    switches go back to their starting values afterwards."""
+    import npeff_ref_amd as d
+
+    yield d.tuning_set
+    d.tuning_reset()
+
+
 @pytest.fixture(scope="session")
 def golden():
     import json

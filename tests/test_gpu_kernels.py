@@ -107,11 +107,11 @@ def test_xg_mu(rows, r):
 
 @pytest.mark.parametrize("split", ["1", "0"])
 @pytest.mark.parametrize("rows", [64, 95, 4100, 70001, 300033])
-def test_xg_mu_gram_fused(rows, split, monkeypatch):
+def test_xg_mu_gram_fused(rows, split, tune):
     """Rank 128, update and Gram matrix of the result in one pass: on the bf16 matrix cores with
     every operand split in three (default) and on the fp32 ones.  Both must meet the fp32 bar;
     the operands span 12 decades and hold zeros, so the split's low parts matter."""
-    monkeypatch.setenv("DNPEFF_SPLIT_BF16", split)
+    tune("split_bf16", float(split))
     r = 128
     rng = np.random.default_rng(rows)
     X = (rng.random((rows, r)) * 10.0 ** rng.uniform(-6, 0, (rows, r))).astype(np.float32)
@@ -176,9 +176,9 @@ def test_spsp_dense(r):
 
 
 @pytest.mark.parametrize("slices,r", [(2, 128), (4, 256), (8, 512), (4, 64)])
-def test_spmm_t_component_slices(slices, r, monkeypatch):
+def test_spmm_t_component_slices(slices, r, tune):
     """The sliced launch of A^T W (one slice of the components per workgroup)."""
-    monkeypatch.setenv("DNPEFF_SPMM_T_SLICES", str(slices))
+    tune("spmm_t_slices", slices)
     rng = np.random.default_rng(slices + r)
     n, m = 3000, 30000
     rowptr, colind, vals, _ = d.synth_pef_host(n, m, k_fixed=300, zipf_s=1.1, seed=7)
@@ -238,7 +238,7 @@ def _hot_column_matrix(rng, n, m, hot, k_tail, dup=False):
 def test_dense_head_products(n, m, hot, r):
     """Columns held by many rows move to a dense block; A H^T and A^T W stay the same sums."""
     rng = np.random.default_rng(n + r)
-    rp, ci, va, hot_cols = _hot_column_matrix(rng, n, m, hot, 40, dup=(r == 64))
+    rp, ci, va, hot_cols = _hot_column_matrix(rng, n, m, hot, 40)
     A = d.Csr.from_host(rp, ci, va, m)
     H = rng.random((m, r)).astype(np.float32)
     W = rng.random((n, r)).astype(np.float32)
@@ -269,6 +269,42 @@ def test_dense_head_products(n, m, hot, r):
     A.close()
 
 
+def test_duplicate_entries_are_refused_by_the_products():
+    """A row that holds a column twice has no deterministic transposed copy: the loader still
+    takes the matrix (the reference's loader does not look either), the products refuse it."""
+    rng = np.random.default_rng(8)
+    rp, ci, va, _ = _hot_column_matrix(rng, 200, 3000, 30, 40, dup=True)
+    A = d.Csr.from_host(rp, ci, va, 3000)
+    assert np.array_equal(A.download()[1], ci)
+    with pytest.raises(d.DnpeffError, match="duplicate"):
+        A.build_transpose()
+    H = d.DeviceArray.from_numpy(rng.random((3000, 64)).astype(np.float32))
+    with pytest.raises(d.DnpeffError, match="duplicate"):
+        d.op_spmm_n(A, 64, H, d.DeviceArray((200, 64)))
+    A.close()
+
+
+def test_spmm_t_is_bit_identical_on_a_rerun():
+    rng = np.random.default_rng(21)
+    n, m, r = 2000, 20000, 128
+    rowptr, colind, vals, _ = d.synth_pef_host(n, m, k_fixed=400, zipf_s=1.1, seed=5)
+    A = d.Csr.from_host(rowptr, colind, vals, m)
+    dW = d.DeviceArray.from_numpy(rng.random((n, r)).astype(np.float32))
+    T1, T2 = d.DeviceArray((m, r)), d.DeviceArray((m, r))
+    d.op_spmm_t(A, r, dW, T1)
+    d.op_spmm_t(A, r, dW, T2)
+    d.sync()
+    assert np.array_equal(T1.numpy(), T2.numpy())
+    A.close()
+    # a second build of the transposed copy gives the same arrays
+    B = d.Csr.from_host(rowptr, colind, vals, m)
+    A2 = d.Csr.from_host(rowptr, colind, vals, m)
+    for x, y in zip(B.download_transpose(), A2.download_transpose()):
+        assert np.array_equal(x, y)
+    B.close()
+    A2.close()
+
+
 def test_dense_head_needs_rank_multiple_of_4():
     rng = np.random.default_rng(3)
     rp, ci, va, _ = _hot_column_matrix(rng, 100, 1000, 20, 10)
@@ -282,10 +318,10 @@ def test_dense_head_needs_rank_multiple_of_4():
 
 @pytest.mark.parametrize("panels,r,n,m,maxk", [(8, 128, 130, 5000, 3000), (37, 64, 61, 900, 400), (256, 50, 300, 20000, 700), (512, 32, 40, 30000, 2000),
                                                (2, 16, 5, 40, 30)])
-def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
+def test_spmm_n_column_panels(panels, r, n, m, maxk, tune):
     """Entries regrouped by column panel, one wave per (row, panel) segment: same sums, same bits
     on every run, empty rows and empty segments included."""
-    monkeypatch.setenv("DNPEFF_PANELS", str(panels))
+    tune("panels", panels)
     rng = np.random.default_rng(panels + r)
     rp, ci, va = random_csr(rng, n, m, maxk, empty_rows={1, n - 1})
     A = d.Csr.from_host(rp, ci, va, m)
@@ -305,7 +341,7 @@ def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
     assert _rel(dT.numpy(), orc.spmm_t_f64(rp, ci, va, m, W)) < TOL
     assert np.array_equal(A.download()[1], ci)
     # without panels: the chunked path again
-    monkeypatch.setenv("DNPEFF_PANELS", "0")
+    tune("panels", 0)
     d.op_spmm_n(A, r, dH, dN)
     assert _rel(dN.numpy(), N64) < TOL
     A.close()
@@ -323,14 +359,14 @@ def test_spmm_n_column_panels(panels, r, n, m, maxk, monkeypatch):
     (32, 150, 3000, 2500, 2, 400 * 128, 4),      # long segments at 8 lane groups (shuffles, no row broadcasts)
     (256, 120, 3000, 2800, 2, 500 * 1024, 6),    # long segments at one lane group (4 rows of 16 lanes)
 ])
-def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, monkeypatch):
+def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, tune):
     """Coarse panels cut into L2-sized pieces that one XCD sweeps for all rows, running sums in
     registers: same sums as the fp64 restatement, same bits on every run, empty rows included; a
     factor that is not 16-byte aligned takes the 4-byte loads."""
-    monkeypatch.setenv("DNPEFF_PANELS", str(panels))
-    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", str(sweep_bytes))
-    monkeypatch.setenv("DNPEFF_SWEEP_MIN", "0")
-    monkeypatch.setenv("DNPEFF_SWEEP_WAVES", str(waves))
+    tune("panels", panels)
+    tune("sweep_bytes", sweep_bytes)
+    tune("sweep_min", 0)
+    tune("sweep_waves", waves)
     rng = np.random.default_rng(r + n)
     rp, ci, va = random_csr(rng, n, m, maxk, empty_rows={0, n // 2})
     A = d.Csr.from_host(rp, ci, va, m)
@@ -350,19 +386,19 @@ def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, monkeypa
     d.op_spmm_n(A, r, view, dN)
     assert (np.abs(dN.numpy() - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
     # workgroups that stop waiting for each other after one poll: same bits
-    monkeypatch.setenv("DNPEFF_SWEEP_SPIN", "1")
+    tune("sweep_spin", 1)
     d.op_spmm_n(A, r, dH, dN)
     assert np.array_equal(dN.numpy(), N)
-    monkeypatch.delenv("DNPEFF_SWEEP_SPIN")
+    tune("sweep_spin", 400)
     # without sweeps: every panel one wave per (row, panel) segment
-    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", "0")
+    tune("sweep_bytes", 0)
     d.op_spmm_n(A, r, dH, dN)
     assert _rel(dN.numpy(), N64) < TOL
     A.close()
 
 
-def test_column_panels_with_dense_head(monkeypatch):
-    monkeypatch.setenv("DNPEFF_PANELS", "16")
+def test_column_panels_with_dense_head(tune):
+    tune("panels", 16)
     rng = np.random.default_rng(11)
     n, m, r = 400, 6000, 128
     rp, ci, va, hot_cols = _hot_column_matrix(rng, n, m, 50, 200)
@@ -390,12 +426,12 @@ def test_threshold_compact_bit_exact(n, div, thr):
 @pytest.mark.parametrize("n,count,k", [(3, 100000, 4096), (2, 5000, 1), (1, 70001, 70001), (4, 30000, 5000),
                                        (1, 3_000_000, 65536)])
 @pytest.mark.parametrize("cap", [None, 0, 9000])
-def test_topk_rows_bit_exact(n, count, k, cap, monkeypatch):
+def test_topk_rows_bit_exact(n, count, k, cap, tune):
     """Device top-k sparsifier vs the full-sort restatement: same values, same indices (ties by
     ascending index), zeros and repeated values included; both the two-read path and the
     exact-threshold path for crowded bins (forced with a zero cap)."""
     if cap is not None:
-        monkeypatch.setenv("DNPEFF_TOPK_FAST_CAP", str(cap))
+        tune("topk_fast_cap", cap)
     rng = np.random.default_rng(count + k)
     x = rng.lognormal(-8, 2, size=(n, count)).astype(np.float32)
     x[0, ::5] = 0.0

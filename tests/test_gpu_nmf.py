@@ -179,7 +179,7 @@ def test_fit_path_first_stage_and_loop():
     H.close()
 
 
-def test_dense_head_run_matches_oracle_and_unsplit_run(monkeypatch):
+def test_dense_head_run_matches_oracle_and_unsplit_run(tune):
     """n >= 1024 rows and r >= 64: dnpeff_nmf_create moves the columns most rows hold into the
     dense block by itself; the run stays within the bar of the fp64 oracle and close to the run
     with the split switched off."""
@@ -192,7 +192,7 @@ def test_dense_head_run_matches_oracle_and_unsplit_run(monkeypatch):
     assert np.all(np.abs(got - losses64) / losses64 < REL)
     nmf.close()
     A.close()
-    monkeypatch.setenv("DNPEFF_DENSE_FILL", "0")
+    tune("dense_fill", 0)
     nmf2, A2, _, (W2, H2), _, hist2, _ = _run_case(n, m_full, k, r, eps, iters, seed)
     assert A2.head_info()[0] == 0
     assert _nrm(W2, W64) < REL and _nrm(H2, H64) < REL
@@ -200,8 +200,8 @@ def test_dense_head_run_matches_oracle_and_unsplit_run(monkeypatch):
     A2.close()
 
 
-def test_column_panel_run_matches_oracle(monkeypatch):
-    monkeypatch.setenv("DNPEFF_PANELS", "12")
+def test_column_panel_run_matches_oracle(tune):
+    tune("panels", 12)
     nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(300, 40000, 2048, 128, 1e-8, 50, seed=5)
     assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
     got = np.array([h[1] for h in hist])
@@ -211,14 +211,14 @@ def test_column_panel_run_matches_oracle(monkeypatch):
 
 
 @pytest.mark.parametrize("r,waves,piece_cols", [(128, 14, 40), (64, 3, 2000)])
-def test_swept_piece_run_matches_oracle(r, waves, piece_cols, monkeypatch):
+def test_swept_piece_run_matches_oracle(r, waves, piece_cols, tune):
     """Column panels cut into small pieces that the XCDs sweep (forced on, any density; at 40
     columns per piece all 6 panels are cut, at 2000 the 3 narrow ones stay whole and both kernels
     share the product): 50 iterations stay within the bar, and a second run gives the same bits."""
-    monkeypatch.setenv("DNPEFF_PANELS", "6")
-    monkeypatch.setenv("DNPEFF_SWEEP_BYTES", str(piece_cols * 4 * r))
-    monkeypatch.setenv("DNPEFF_SWEEP_MIN", "0")
-    monkeypatch.setenv("DNPEFF_SWEEP_WAVES", str(waves))
+    tune("panels", 6)
+    tune("sweep_bytes", piece_cols * 4 * r)
+    tune("sweep_min", 0)
+    tune("sweep_waves", waves)
     nmf, A, _, (W, H), (W64, H64), hist, losses64 = _run_case(300, 40000, 2048, r, 1e-8, 50, seed=9)
     assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
     got = np.array([h[1] for h in hist])
@@ -231,11 +231,11 @@ def test_swept_piece_run_matches_oracle(r, waves, piece_cols, monkeypatch):
     A2.close()
 
 
-def test_ragged_rows_rank_512(monkeypatch):
+def test_ragged_rows_rank_512(tune):
     """Row lengths drawn log-uniformly over two decades (the ragged-row case), r = 512: the tiled
     X G kernel, the tile-pair Gram and the grouped A^T W at their widest, with column panels
     forced on so that short rows leave empty segments."""
-    monkeypatch.setenv("DNPEFF_PANELS", "24")
+    tune("panels", 24)
     n, m_full, r, eps, iters, seed = 260, 60000, 512, 1e-8, 50, 31
     A, norms = d.Csr.synth(n, m_full, k_fixed=0, k_min=16, k_max=4096, zipf_s=1.1, seed=seed)
     A.normalize_rows(norms)
@@ -295,7 +295,7 @@ def test_fit_after_nmf_on_the_same_matrix():
     B.close()
 
 
-def test_fused_gram_in_H_update_matches_the_two_pass_path(monkeypatch):
+def test_fused_gram_in_H_update_matches_the_two_pass_path(tune):
     """r = 128: the H update accumulates H^T H of its own output, the W update uses it; rows past
     the last 64-row tile go through the plain kernels and are added.  Same bar against the oracle
     with the fusion switched off, and the two runs agree far inside it."""
@@ -305,10 +305,89 @@ def test_fused_gram_in_H_update_matches_the_two_pass_path(monkeypatch):
     assert _nrm(W, W64) < REL and _nrm(H, H64) < REL
     nmf.close()
     A.close()
-    monkeypatch.setenv("DNPEFF_FUSED_GRAM", "0")
+    tune("fused_gram", 0)
     nmf2, A2, _, (W2, H2), _, hist2, _ = _run_case(*args, seed=5)
     assert _nrm(W2, W64) < REL and _nrm(H2, H64) < REL
     assert _nrm(W, W2.astype(np.float64)) < 1e-5 and _nrm(H, H2.astype(np.float64)) < 1e-5
     assert abs(hist[-1][1] - hist2[-1][1]) / hist2[-1][1] < 1e-6
     nmf2.close()
     A2.close()
+
+
+def _steps(A, r, seed, steps, consume=False):
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=0, eps=1e-8, seed=seed), consume_matrix=consume)
+    nmf.initialize()
+    nmf.step(steps)
+    d.sync()
+    return nmf
+
+
+@pytest.mark.parametrize("r,n,k,tile_mb", [(256, 1100, 3000, 0.9), (128, 1100, 3000, 0.4), (64, 300, 2000, 0.05),
+                                           (48, 130, 800, 0.03)])
+def test_tiled_H_update_gives_the_same_bits(r, n, k, tile_mb, tune):
+    """The H update on column tiles (A^T W of a tile, then the tile's update written one tile
+    away inside the buffer of H; forced here, used by itself when a second [m, r] array does not
+    fit) against the full-size update: same factors bit for bit after an odd and an even number
+    of steps (H sits at either end of its buffer), dense head and long columns included; the
+    consuming create frees the caller's arrays and changes nothing else."""
+    tune("fused_gram", 0)  # (at rank 128 the fused update sums in another order)
+    seed = 100 + r
+    A, norms = d.Csr.synth(n, 60000, k_fixed=k, zipf_s=1.2, seed=seed)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    ref = _steps(A, r, seed, 3)
+    assert ref.info() == (False, 0)
+    W3, H3 = ref.loadWToHostSync(), ref.loadHToHostSync()
+    ref.step(1)
+    W4, H4, loss4 = ref.loadWToHostSync(), ref.loadHToHostSync(), ref.computeUncachedLoss()
+    ref.close()
+    tune("tiled_h", 1)
+    tune("h_tile_mb", tile_mb)
+    til = _steps(A, r, seed, 3, consume=True)
+    tiled, tile_cols = til.info()
+    assert tiled and tile_cols % 128 == 0 and 2 * tile_cols < A.n_cols
+    if r >= 64 and n >= 1024:
+        assert A.head_info()[0] > 0
+    assert np.array_equal(til.loadWToHostSync(), W3) and np.array_equal(til.loadHToHostSync(), H3)
+    til.step(1)
+    assert np.array_equal(til.loadWToHostSync(), W4) and np.array_equal(til.loadHToHostSync(), H4)
+    assert til.computeUncachedLoss() == loss4
+    # factors loaded from the host go through the same tiles
+    til.set_factors(W3, H3)
+    assert np.array_equal(til.loadHToHostSync(), H3)
+    til.step(1)
+    assert np.array_equal(til.loadHToHostSync(), H4)
+    # the consumed matrix still knows its shape and column map, and refuses to be read back
+    assert len(A.kept_indices()) == A.n_cols
+    if A.head_info()[0] > 0:  # (without head or panels the products read the caller's arrays)
+        with pytest.raises(d.DnpeffError, match="released"):
+            A.download()
+        with pytest.raises(d.DnpeffError, match="released"):
+            A.compact_columns(1)
+    else:
+        assert len(A.download()[1]) == A.nnz
+    til.close()
+    A.close()
+
+
+def test_two_contexts_of_different_rank_on_one_matrix():
+    """A second context (or a single-kernel call) at another rank plans the matrix's work lists
+    and partial-sum buffers again; the first context must notice and still give its own results."""
+    seed = 12
+    A, norms = d.Csr.synth(600, 200000, k_fixed=4000, zipf_s=1.1, seed=seed)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    alone = _steps(A, 128, seed, 2)
+    W_ref, H_ref = alone.loadWToHostSync(), alone.loadHToHostSync()
+    alone.close()
+    big = _steps(A, 128, seed, 1)
+    small = _steps(A, 32, seed, 1)  # plans the matrix for rank 32: smaller partial sums
+    big.step(1)                     # rank 128 again
+    small.step(1)
+    assert np.array_equal(big.loadWToHostSync(), W_ref) and np.array_equal(big.loadHToHostSync(), H_ref)
+    small_alone = _steps(A, 32, seed, 2)
+    assert np.array_equal(small.loadWToHostSync(), small_alone.loadWToHostSync())
+    small_alone.close()
+    big.close()
+    small.close()
+    A.close()
