@@ -161,6 +161,17 @@ int dnpeff_csr_head_info(const dnpeff_csr* A, int64_t* n_dense, int64_t* nnz_spa
 /* Copy the transposed CSR back: colptr[n_cols+1], rowind[nnz], vals[nnz]. */
 int dnpeff_csr_download_transpose(dnpeff_csr* A, int64_t* colptr, int32_t* rowind, float* vals);
 
+/* One row / one column of the matrix as the products hold it (dense head block plus sparse
+ * part), to the host: *count receives the number of entries; cols/rows and vals (may be NULL
+ * to ask for the count only) must hold cap >= count entries.  Order: head entries first, then
+ * the sparse part's (a row: in its stored order; a column: ascending rows).  Works on a matrix
+ * consumed by dnpeff_nmf_create_ex.  Counterpart of the inspection helpers of
+ * cc/cuda_d_npeff/src/util/matrices.h:258-324 (asDenseMatrix / areEqual), for validation. */
+int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* count, int32_t* cols,
+                       float* vals);
+int dnpeff_csr_get_column(dnpeff_csr* A, int64_t col, int64_t cap, int64_t* count, int32_t* rows,
+                          float* vals);
+
 /* Release the arrays that only dnpeff_op_spmm_n / dnpeff_nmf_* need (row-major
  * copy) or only spmm_t needs (transposed copy).  which: 1 = row-major copy,
  * 2 = transposed copy. */
@@ -196,6 +207,14 @@ int dnpeff_synth_pef_host(int64_t n_rows, int64_t n_cols, int64_t k_fixed,
                           double mu, double sigma, uint64_t seed,
                           int64_t* rowptr, int32_t* colind, float* vals,
                           float* norms);
+
+/* Rows [row0, row0 + n_rows) of the matrix that dnpeff_synth_pef makes for the same other
+ * arguments (rows are keyed by their absolute number), for checks of a large device-made matrix
+ * on sampled rows; rowptr[n_rows + 1] is relative to the first of these rows. */
+int dnpeff_synth_pef_host_rows(int64_t row0, int64_t n_rows, int64_t n_cols, int64_t k_fixed,
+                               int64_t k_min, int64_t k_max, double zipf_s, double mu, double sigma,
+                               uint64_t seed, int64_t* rowptr, int32_t* colind, float* vals,
+                               float* norms);
 
 /* U[0,1) initial factor value of logical element (row, col) of matrix
  * matrix_id (0 = W [n, r], 1 = H [r, m]); host mirror of the device
@@ -257,6 +276,14 @@ int dnpeff_nmf_loss(dnpeff_nmf* nmf, double* out);
 
 /* The three terms of the loss: ||A||^2, <H,(W^T W)H>, <W^T A,H>. */
 int dnpeff_nmf_loss_terms(dnpeff_nmf* nmf, double* sq_norm_A, double* pos, double* neg);
+
+/* Consistency of the two sparse products on the current factors: <A H^T, W> computed through
+ * the row-ordered structures (the kernels of the W update) and <A^T W, H> through the
+ * column-ordered ones (the kernels of the H update, tile by tile when H is updated so).  The
+ * two are the same number, the third term of the loss (multi_mu_dense_factors_nmf1.h:270-273);
+ * an entry lost, doubled or misplaced in either copy of the matrix makes them differ.  Costs one
+ * A H^T and one A^T W; does not change the factors. */
+int dnpeff_nmf_check_products(dnpeff_nmf* nmf, double* via_rows, double* via_columns);
 
 /* Copy the factors to the host in the output-file layout: W [n, r] row-major
  * (loadWToHostSync + toRowMajor_inPlace, nmf1.h:207-220, matrices.h:49-62),
@@ -335,6 +362,11 @@ int dnpeff_op_spmm_n(dnpeff_csr* A, int r, const float* H_mr, float* N_nr);
  * cusparseSpMM(T, T) at device_contexts1.h:260-265,301. */
 int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 
+/* Rows [col0, col1) of A^T W into T_tile [col1 - col0, r]: the product on a column tile, as the
+ * tiled H update of dnpeff_nmf_update_H forms it. */
+int dnpeff_op_spmm_t_tile(dnpeff_csr* A, int r, const float* W_nr, int64_t col0, int64_t col1,
+                          float* T_tile);
+
 /* Keeps the elements with x[i] / divisor >= threshold (fp32 division, then the comparison):
  * idx_out receives their positions in ascending order, val_out the divided values, *n_kept
  * (host) their number; idx_out and val_out are device buffers of `count` elements.  One row of
@@ -388,6 +420,10 @@ int dnpeff_op_dot(int64_t count, const float* x, const float* y, double* out_hos
  * transposed copy is built if missing.  Partitioned_SpSpMatmul_ToDense
  * (cc/cuda_d_npeff/src/cuda/ops/spsp_matmul.h:95-131). */
 int dnpeff_op_spsp_dense(dnpeff_csr* A, dnpeff_csr* B, float* out_nr);
+
+/* out[k, :] = X[rows_dev[k], :] for k < count: rows of r floats picked from a device array by a
+ * device index list (test and validation helper: sampled rows of a factor). */
+int dnpeff_op_gather_rows(int64_t count, int r, const float* X, const int32_t* rows_dev, float* out);
 
 /* dst[i] = src[i], i < count: a plain streaming copy of known size, the yardstick
  * that hardware-counter readings (FETCH_SIZE, WRITE_SIZE) are scaled by. */

@@ -24,6 +24,8 @@ from .binding import (  # noqa: F401
     size_of_split,
     uniform_at,
     synth_pef_host,
+    synth_pef_host_rows,
+    gather_rows,
     KERNEL_CLASSES,
     sync,
     device_info,

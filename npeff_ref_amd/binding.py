@@ -77,6 +77,13 @@ SIGNATURES = {
         C.c_int,
         [_i64, _i64, _i64, _i64, _i64, _f64, _f64, _f64, _u64, _p, _p, _p, _p],
     ),
+    "dnpeff_synth_pef_host_rows": (
+        C.c_int,
+        [_i64, _i64, _i64, _i64, _i64, _i64, _f64, _f64, _f64, _u64, _p, _p, _p, _p],
+    ),
+    "dnpeff_csr_get_row": (C.c_int, [_p, _i64, _i64, C.POINTER(_i64), _p, _p]),
+    "dnpeff_csr_get_column": (C.c_int, [_p, _i64, _i64, C.POINTER(_i64), _p, _p]),
+    "dnpeff_op_gather_rows": (C.c_int, [_i64, C.c_int, _p, _p, _p]),
     "dnpeff_uniform_at": (_f32, [_u64, C.c_int, _i64, _i64, _i64]),
     "dnpeff_nmf_create": (C.c_int, [_p, C.c_int, _f32, _i64, _pp]),
     "dnpeff_nmf_create_ex": (C.c_int, [_p, C.c_int, _f32, _i64, C.c_uint, _pp]),
@@ -88,6 +95,7 @@ SIGNATURES = {
     "dnpeff_nmf_update_H": (C.c_int, [_p]),
     "dnpeff_nmf_loss": (C.c_int, [_p, C.POINTER(_f64)]),
     "dnpeff_nmf_loss_terms": (C.c_int, [_p, C.POINTER(_f64), C.POINTER(_f64), C.POINTER(_f64)]),
+    "dnpeff_nmf_check_products": (C.c_int, [_p, C.POINTER(_f64), C.POINTER(_f64)]),
     "dnpeff_nmf_get_W": (C.c_int, [_p, _p]),
     "dnpeff_nmf_get_H": (C.c_int, [_p, _p]),
     "dnpeff_nmf_device_factors": (C.c_int, [_p, _pp, _pp]),
@@ -105,6 +113,7 @@ SIGNATURES = {
     "dnpeff_op_mu": (C.c_int, [_i64, _p, _p, _p, _f32]),
     "dnpeff_op_spmm_n": (C.c_int, [_p, C.c_int, _p, _p]),
     "dnpeff_op_spmm_t": (C.c_int, [_p, C.c_int, _p, _p]),
+    "dnpeff_op_spmm_t_tile": (C.c_int, [_p, C.c_int, _p, _i64, _i64, _p]),
     "dnpeff_op_gram": (C.c_int, [_i64, C.c_int, _p, _p]),
     "dnpeff_op_gram_static": (C.c_int, [_i64, C.c_int, _p, _p]),
     "dnpeff_op_xg_mu": (C.c_int, [_i64, C.c_int, _p, _p, _p, _f32, _p, _p]),
@@ -198,6 +207,33 @@ def synth_pef_host(n_rows, n_cols, k_fixed=0, k_min=0, k_max=0, zipf_s=1.1, mu=-
     norms = np.zeros(n_rows, dtype=np.float32)
     _check(lib.dnpeff_synth_pef_host(*args, _ptr(rowptr), _ptr(colind), _ptr(vals), _ptr(norms)))
     return rowptr, colind, vals, norms
+
+
+def synth_pef_host_rows(row0, n_rows, n_cols, k_fixed=0, k_min=0, k_max=0, zipf_s=1.1, mu=-8.0, sigma=2.0,
+                        seed=0):
+    """Rows [row0, row0 + n_rows) of the device generator's matrix, made on the host."""
+    rowptr = np.zeros(n_rows + 1, dtype=np.int64)
+    args = (row0, n_rows, n_cols, k_fixed, k_min, k_max, zipf_s, mu, sigma, seed & 0xFFFFFFFFFFFFFFFF)
+    _check(lib.dnpeff_synth_pef_host_rows(*args, _ptr(rowptr), None, None, None))
+    nnz = int(rowptr[-1])
+    colind = np.zeros(nnz, dtype=np.int32)
+    vals = np.zeros(nnz, dtype=np.float32)
+    norms = np.zeros(n_rows, dtype=np.float32)
+    _check(lib.dnpeff_synth_pef_host_rows(*args, _ptr(rowptr), _ptr(colind), _ptr(vals), _ptr(norms)))
+    return rowptr, colind, vals, norms
+
+
+def gather_rows(dev_ptr, r: int, rows) -> np.ndarray:
+    """Rows `rows` of a device array of r floats per row, as a numpy array."""
+    rows = np.ascontiguousarray(rows, dtype=np.int32)
+    idx = DeviceArray.from_numpy(rows, dtype=np.int32)
+    out = DeviceArray((len(rows), r))
+    _check(lib.dnpeff_op_gather_rows(len(rows), r, C.c_void_p(dev_ptr), idx.ptr, out.ptr))
+    sync()
+    res = out.numpy()
+    idx.free()
+    out.free()
+    return res
 
 
 class DeviceArray:
@@ -408,6 +444,24 @@ class Csr:
         _check(lib.dnpeff_csr_kept_indices(self._h, _ptr(out)))
         return out
 
+    def get_row(self, row: int):
+        """(cols, vals) of one row as the products hold it (works on a consumed matrix)."""
+        cnt = _i64(0)
+        _check(lib.dnpeff_csr_get_row(self._h, row, 0, C.byref(cnt), None, None))
+        cols = np.zeros(cnt.value, dtype=np.int32)
+        vals = np.zeros(cnt.value, dtype=np.float32)
+        _check(lib.dnpeff_csr_get_row(self._h, row, cnt.value, C.byref(cnt), _ptr(cols), _ptr(vals)))
+        return cols, vals
+
+    def get_column(self, col: int):
+        """(rows, vals) of one column as the products hold it."""
+        cnt = _i64(0)
+        _check(lib.dnpeff_csr_get_column(self._h, col, 0, C.byref(cnt), None, None))
+        rows = np.zeros(cnt.value, dtype=np.int32)
+        vals = np.zeros(cnt.value, dtype=np.float32)
+        _check(lib.dnpeff_csr_get_column(self._h, col, cnt.value, C.byref(cnt), _ptr(rows), _ptr(vals)))
+        return rows, vals
+
     def sq_norm(self) -> float:
         v = _f64(0)
         _check(lib.dnpeff_csr_sq_norm(self._h, C.byref(v)))
@@ -543,6 +597,12 @@ class MuNmf:
         a, p, q = _f64(0), _f64(0), _f64(0)
         _check(lib.dnpeff_nmf_loss_terms(self._h, C.byref(a), C.byref(p), C.byref(q)))
         return a.value, p.value, q.value
+
+    def check_products(self):
+        """(<A H^T, W> via the row-ordered kernels, <A^T W, H> via the column-ordered ones)."""
+        a, b = _f64(0), _f64(0)
+        _check(lib.dnpeff_nmf_check_products(self._h, C.byref(a), C.byref(b)))
+        return a.value, b.value
 
     def loadWToHostSync(self) -> np.ndarray:
         """W as [n, r] row-major (after the reference's toRowMajor_inPlace)."""

@@ -441,6 +441,38 @@ DN_API int dnpeff_nmf_loss_terms(dnpeff_nmf* h, double* sq_norm_A, double* pos, 
   return 0;
 }
 
+DN_API int dnpeff_nmf_check_products(dnpeff_nmf* h, double* via_rows, double* via_columns) {
+  clear_error();
+  DN_CHECK(h && via_rows && via_columns, "NULL argument");
+  dnpeff_csr* A = h->A;
+  DN_TRY(products_for(h));
+  // <A H^T, W> through the row-ordered structures
+  DN_TRY(launch_spmm_n(A, h->r, h->H));
+  DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
+  h->nw_valid = true;
+  DN_TRY(launch_dot(h->n * h->r, h->Nw, h->W, h->dot_ws, h->dot_ws + DOT_BLOCKS));
+  DN_HIP(hipStreamSynchronize(stream()));
+  DN_HIP(hipMemcpy(via_rows, h->dot_ws + DOT_BLOCKS, sizeof(double), hipMemcpyDeviceToHost));
+  // <A^T W, H> through the column-ordered ones (S is free between two H updates)
+  double sum = 0.0;
+  const int64_t step = h->tiled ? h->tile_cols : h->m;
+  if (h->tiled) DN_TRY(launch_head_t_product(A, h->r, h->W));
+  for (int64_t c0 = 0; c0 < h->m; c0 += step) {
+    const int64_t c1 = c0 + step < h->m ? c0 + step : h->m;
+    if (h->tiled)
+      DN_TRY(launch_spmm_t_tile(A, h->r, h->W, c0, c1, h->S));
+    else
+      DN_TRY(launch_spmm_t(A, h->r, h->W, h->S));
+    DN_TRY(launch_dot((c1 - c0) * h->r, h->S, h->H + c0 * h->r, h->dot_ws, h->dot_ws + DOT_BLOCKS + 1));
+    double part = 0.0;
+    DN_HIP(hipStreamSynchronize(stream()));
+    DN_HIP(hipMemcpy(&part, h->dot_ws + DOT_BLOCKS + 1, sizeof(double), hipMemcpyDeviceToHost));
+    sum += part;
+  }
+  *via_columns = sum;
+  return 0;
+}
+
 DN_API int dnpeff_nmf_loss(dnpeff_nmf* nmf, double* out) {
   DN_CHECK(out != nullptr, "out is NULL");
   double a, p, q;

@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstdlib>
 
+#include <algorithm>
 #include <cctype>
 #include <cstdarg>
 #include <cstring>
@@ -1357,6 +1358,116 @@ DN_API int dnpeff_csr_download_transpose(dnpeff_csr* A, int64_t* colptr, int32_t
     DN_HIP(hipMemcpy(rowind, A->rowind, sizeof(int32_t) * A->nnz, hipMemcpyDeviceToHost));
   if (vals && A->nnz)
     DN_HIP(hipMemcpy(vals, A->tvals, sizeof(float) * A->nnz, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+// out[k] = X[rows[k]] for k < count (rows of r floats)
+__global__ void __launch_bounds__(256)
+    k_gather_rows(const float* __restrict__ X, const int32_t* __restrict__ rows, int64_t count, int r,
+                  float* __restrict__ out) {
+  const int64_t total = count * r, stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride)
+    out[e] = X[(int64_t)rows[e / r] * r + e % r];
+}
+
+DN_API int dnpeff_op_gather_rows(int64_t count, int r, const float* X, const int32_t* rows_dev,
+                                 float* out) {
+  clear_error();
+  DN_CHECK(count >= 0 && r >= 1, "bad arguments");
+  if (count == 0) return 0;
+  DN_CHECK(X && rows_dev && out, "NULL argument");
+  hipLaunchKernelGGL(k_gather_rows, dim3(grid_for(count * r)), dim3(256), 0, stream(), X, rows_dev,
+                     count, r, out);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+// Entries of one row / one column of the matrix as the products hold it: the dense head's block
+// plus the sparse part (its regrouped or plain row-major copy, its transposed copy).
+DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* count, int32_t* cols,
+                              float* vals) {
+  clear_error();
+  DN_CHECK(A && count, "NULL argument");
+  DN_CHECK(row >= 0 && row < A->n_rows, "row %lld outside [0, %lld)", (long long)row,
+           (long long)A->n_rows);
+  DN_HIP(hipStreamSynchronize(stream()));
+  const dnpeff_csr* S = sparse_part(A);
+  DN_CHECK(S->rowptr != nullptr, "matrix has no row offsets");
+  int64_t e[2];
+  DN_HIP(hipMemcpy(e, S->rowptr + row, sizeof(e), hipMemcpyDeviceToHost));
+  const int32_t* src_c = S->colind ? S->colind : S->pcol;
+  const float* src_v = S->vals ? S->vals : S->pval;
+  DN_CHECK(e[1] == e[0] || (src_c && src_v), "matrix holds no row-major copy of its sparse part");
+  int64_t got = e[1] - e[0];
+  std::vector<float> head_row;
+  std::vector<int32_t> head_cols;
+  if (A->head.n_d) {
+    head_row.resize((size_t)A->head.n_d);
+    head_cols.resize((size_t)A->head.n_d);
+    DN_HIP(hipMemcpy(head_row.data(), A->head.rm + row * A->head.n_d_pad, sizeof(float) * A->head.n_d,
+                     hipMemcpyDeviceToHost));
+    DN_HIP(hipMemcpy(head_cols.data(), A->head.cols, sizeof(int32_t) * A->head.n_d,
+                     hipMemcpyDeviceToHost));
+    for (float v : head_row) got += v != 0.0f;
+  }
+  *count = got;
+  if (!cols || !vals) return 0;
+  DN_CHECK(cap >= got, "row %lld holds %lld entries, the buffers %lld", (long long)row, (long long)got,
+           (long long)cap);
+  int64_t w = 0;
+  for (size_t k = 0; k < head_row.size(); k++)
+    if (head_row[k] != 0.0f) {
+      cols[w] = head_cols[k];
+      vals[w++] = head_row[k];
+    }
+  if (e[1] > e[0]) {
+    DN_HIP(hipMemcpy(cols + w, src_c + e[0], sizeof(int32_t) * (e[1] - e[0]), hipMemcpyDeviceToHost));
+    DN_HIP(hipMemcpy(vals + w, src_v + e[0], sizeof(float) * (e[1] - e[0]), hipMemcpyDeviceToHost));
+  }
+  return 0;
+}
+
+DN_API int dnpeff_csr_get_column(dnpeff_csr* A, int64_t col, int64_t cap, int64_t* count,
+                                 int32_t* rows, float* vals) {
+  clear_error();
+  DN_CHECK(A && count, "NULL argument");
+  DN_CHECK(col >= 0 && col < A->n_cols, "column %lld outside [0, %lld)", (long long)col,
+           (long long)A->n_cols);
+  dnpeff_csr* S = sparse_part(A);
+  DN_TRY(dnpeff_csr_build_transpose(S));
+  DN_TRY(csr_tile_lists(A));
+  DN_HIP(hipStreamSynchronize(stream()));
+  const std::vector<int32_t>& hc = A->h_head_cols;
+  const auto it = std::lower_bound(hc.begin(), hc.end(), (int32_t)col);
+  if (it != hc.end() && *it == (int32_t)col) {  // a column of the dense head
+    const int64_t k = it - hc.begin();
+    std::vector<float> c((size_t)A->n_rows);
+    DN_HIP(hipMemcpy(c.data(), A->head.cm + k * A->head.n_pad, sizeof(float) * A->n_rows,
+                     hipMemcpyDeviceToHost));
+    int64_t got = 0;
+    for (float v : c) got += v != 0.0f;
+    *count = got;
+    if (!rows || !vals) return 0;
+    DN_CHECK(cap >= got, "column %lld holds %lld entries, the buffers %lld", (long long)col,
+             (long long)got, (long long)cap);
+    int64_t w = 0;
+    for (int64_t i = 0; i < A->n_rows; i++)
+      if (c[(size_t)i] != 0.0f) {
+        rows[w] = (int32_t)i;
+        vals[w++] = c[(size_t)i];
+      }
+    return 0;
+  }
+  int64_t p[2];
+  DN_HIP(hipMemcpy(p, S->colptr + col, sizeof(p), hipMemcpyDeviceToHost));
+  *count = p[1] - p[0];
+  if (!rows || !vals) return 0;
+  DN_CHECK(cap >= p[1] - p[0], "column %lld holds %lld entries, the buffers %lld", (long long)col,
+           (long long)(p[1] - p[0]), (long long)cap);
+  if (p[1] > p[0]) {
+    DN_HIP(hipMemcpy(rows, S->rowind + p[0], sizeof(int32_t) * (p[1] - p[0]), hipMemcpyDeviceToHost));
+    DN_HIP(hipMemcpy(vals, S->tvals + p[0], sizeof(float) * (p[1] - p[0]), hipMemcpyDeviceToHost));
+  }
   return 0;
 }
 

@@ -1248,6 +1248,16 @@ DN_API int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr
   return launch_spmm_t(A, r, W_nr, T_mr);
 }
 
+DN_API int dnpeff_op_spmm_t_tile(dnpeff_csr* A, int r, const float* W_nr, int64_t col0, int64_t col1,
+                                 float* T_tile) {
+  clear_error();
+  DN_CHECK(A && W_nr && T_tile, "NULL argument");
+  DN_TRY(csr_ensure_products(A, r));
+  DN_TRY(csr_tile_lists(A));
+  DN_TRY(launch_head_t_product(A, r, W_nr));
+  return launch_spmm_t_tile(A, r, W_nr, col0, col1, T_tile);
+}
+
 DN_API int dnpeff_op_spsp_dense(dnpeff_csr* A, dnpeff_csr* B, float* out_nr) {
   clear_error();
   DN_CHECK(A && B && out_nr, "NULL argument");

@@ -214,17 +214,15 @@ DN_API int dnpeff_synth_pef(int64_t n_rows, int64_t n_cols, int64_t k_fixed, int
   return 0;
 }
 
-DN_API int dnpeff_synth_pef_host(int64_t n_rows, int64_t n_cols, int64_t k_fixed, int64_t k_min,
-                                 int64_t k_max, double zipf_s, double mu, double sigma,
-                                 uint64_t seed, int64_t* rowptr, int32_t* colind, float* vals,
-                                 float* norms) {
-  clear_error();
-  DN_TRY(validate_synth(n_rows, n_cols, k_fixed, k_min, k_max, zipf_s));
+// rows [row0, row0 + n_rows) of the matrix that dnpeff_synth_pef makes for the same arguments
+static int synth_host_rows(int64_t row0, int64_t n_rows, int64_t n_cols, int64_t k_fixed,
+                           int64_t k_min, int64_t k_max, double zipf_s, double mu, double sigma,
+                           uint64_t seed, int64_t* rowptr, int32_t* colind, float* vals, float* norms) {
   DN_CHECK(rowptr != nullptr, "rowptr is NULL");
   rowptr[0] = 0;
   int64_t kmax_eff = 0;
   for (int64_t i = 0; i < n_rows; i++) {
-    int64_t k = dn_row_length(seed, (uint64_t)i, k_fixed, k_min, k_max);
+    int64_t k = dn_row_length(seed, (uint64_t)(row0 + i), k_fixed, k_min, k_max);
     rowptr[i + 1] = rowptr[i] + k;
     if (k > kmax_eff) kmax_eff = k;
   }
@@ -236,13 +234,14 @@ DN_API int dnpeff_synth_pef_host(int64_t n_rows, int64_t n_cols, int64_t k_fixed
   while (cap < 2 * (uint64_t)(kmax_eff + 256)) cap <<= 1;
   std::vector<uint64_t> table(cap);
   const uint64_t mask = cap - 1;
-  for (int64_t row = 0; row < n_rows; row++) {
-    const int64_t base = rowptr[row], k = rowptr[row + 1] - base;
+  for (int64_t i = 0; i < n_rows; i++) {
+    const uint64_t row = (uint64_t)(row0 + i);
+    const int64_t base = rowptr[i], k = rowptr[i + 1] - base;
     std::fill(table.begin(), table.end(), SLOT_EMPTY);
     int64_t count = 0;
     const uint64_t budget = draw_budget(k);
     for (uint64_t t = 0; count < k && t < budget; t++) {
-      const uint64_t id = (uint64_t)dn_zipf_draw(&z, seed, (uint64_t)row, t);
+      const uint64_t id = (uint64_t)dn_zipf_draw(&z, seed, row, t);
       uint64_t slot = slot_hash(id) & mask;
       bool seen = false;
       while (table[slot] != SLOT_EMPTY) {
@@ -256,11 +255,32 @@ DN_API int dnpeff_synth_pef_host(int64_t n_rows, int64_t n_cols, int64_t k_fixed
     DN_CHECK(count == k, "row %lld exhausted its draw budget", (long long)row);
     double s = 0.0;
     for (int64_t p = 0; p < k; p++) {
-      float v = dn_lognormal_at(seed, (uint64_t)row, (uint64_t)p, mu, sigma);
+      float v = dn_lognormal_at(seed, row, (uint64_t)p, mu, sigma);
       vals[base + p] = v;
       s = fma((double)v, (double)v, s);
     }
-    if (norms) norms[row] = (float)sqrt(s);
+    if (norms) norms[i] = (float)sqrt(s);
   }
   return 0;
+}
+
+DN_API int dnpeff_synth_pef_host(int64_t n_rows, int64_t n_cols, int64_t k_fixed, int64_t k_min,
+                                 int64_t k_max, double zipf_s, double mu, double sigma,
+                                 uint64_t seed, int64_t* rowptr, int32_t* colind, float* vals,
+                                 float* norms) {
+  clear_error();
+  DN_TRY(validate_synth(n_rows, n_cols, k_fixed, k_min, k_max, zipf_s));
+  return synth_host_rows(0, n_rows, n_cols, k_fixed, k_min, k_max, zipf_s, mu, sigma, seed, rowptr,
+                         colind, vals, norms);
+}
+
+DN_API int dnpeff_synth_pef_host_rows(int64_t row0, int64_t n_rows, int64_t n_cols, int64_t k_fixed,
+                                      int64_t k_min, int64_t k_max, double zipf_s, double mu,
+                                      double sigma, uint64_t seed, int64_t* rowptr, int32_t* colind,
+                                      float* vals, float* norms) {
+  clear_error();
+  DN_CHECK(row0 >= 0, "row0 is negative");
+  DN_TRY(validate_synth(row0 + n_rows, n_cols, k_fixed, k_min, k_max, zipf_s));
+  return synth_host_rows(row0, n_rows, n_cols, k_fixed, k_min, k_max, zipf_s, mu, sigma, seed, rowptr,
+                         colind, vals, norms);
 }
