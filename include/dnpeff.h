@@ -358,6 +358,13 @@ int dnpeff_op_mu(int64_t count, float* F, const float* num, const float* den, fl
  * device_contexts1.h:255-258,317. */
 int dnpeff_op_spmm_n(dnpeff_csr* A, int r, const float* H_mr, float* N_nr);
 
+/* The same product with the work decomposition of the sparse part chosen by the caller, for
+ * comparisons on ragged rows: 0 = as planned (column panels and swept pieces where the factor
+ * is large, else row chunks), 1 = one wavefront per row, 2 = chunks of 2048 entries of a row with
+ * a second pass over the chunk sums (with rows of 1024 entries and more this is the merge-path
+ * split up to the last, shorter chunk of each row).  1 and 2 need the row-major arrays. */
+int dnpeff_op_spmm_n_variant(dnpeff_csr* A, int r, const float* H_mr, float* N_nr, int variant);
+
 /* T[m, r] = A^T W with W [n, r]; needs dnpeff_csr_build_transpose.
  * cusparseSpMM(T, T) at device_contexts1.h:260-265,301. */
 int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr);

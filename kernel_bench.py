@@ -2,8 +2,8 @@
 """Times one kernel of the library through its C-ABI entry point (dnpeff_op_*), for profiling
 with rocprofv3.
 
-    python3 npeff_ref_amd/kernel_bench.py --op xg_mu --rows 8000000 --rank 128 --iters 5
-    python3 npeff_ref_amd/kernel_bench.py --op spmm_n --n 10000 --m-full 110000000 --k 65536 --rank 128
+    python3 kernel_bench.py --op xg_mu --rows 8000000 --rank 128 --iters 5
+    python3 kernel_bench.py --op spmm_n --n 10000 --m-full 110000000 --k 65536 --rank 128
 
 Dense ops (mu, gram, xg_mu, copy) run on uniform random [rows, rank] operands; sparse ops
 (spmm_n, spmm_t) on a synthetic PEF matrix (Zipf columns, compacted).  `copy` is a plain device
@@ -17,7 +17,7 @@ import time
 
 import numpy as np
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 import npeff_ref_amd as d  # noqa: E402
 

@@ -112,6 +112,7 @@ SIGNATURES = {
     "dnpeff_fit_destroy": (C.c_int, [_p]),
     "dnpeff_op_mu": (C.c_int, [_i64, _p, _p, _p, _f32]),
     "dnpeff_op_spmm_n": (C.c_int, [_p, C.c_int, _p, _p]),
+    "dnpeff_op_spmm_n_variant": (C.c_int, [_p, C.c_int, _p, _p, C.c_int]),
     "dnpeff_op_spmm_t": (C.c_int, [_p, C.c_int, _p, _p]),
     "dnpeff_op_spmm_t_tile": (C.c_int, [_p, C.c_int, _p, _i64, _i64, _p]),
     "dnpeff_op_gram": (C.c_int, [_i64, C.c_int, _p, _p]),

@@ -227,6 +227,23 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// One wave per row, the whole row: the plain row-per-wavefront decomposition, kept for the
+// comparison of work decompositions on ragged rows (a long row then holds its wave for as long
+// as its length says, while the waves of short rows have long finished).
+template <class GT>
+__global__ void __launch_bounds__(256)
+    k_spmm_n_rowwave(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
+                     const float* __restrict__ vals, int64_t n_rows, int r,
+                     const float* __restrict__ H, float* __restrict__ N) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= n_rows) return;
+  GT g;
+  g.init(lane, r);
+  g.run(colind, vals, rowptr[row], rowptr[row + 1], H, r);
+  g.store(N + row * r);
+}
+
 // ---------------------------------------------------------------------------
 // Column panels.  When H is far larger than the caches, every gathered row of H comes from
 // HBM unless the workgroups running at one time gather from the same part of H.  The entries of
@@ -1246,6 +1263,49 @@ DN_API int dnpeff_op_spmm_t(dnpeff_csr* A, int r, const float* W_nr, float* T_mr
   DN_CHECK(A && W_nr && T_mr, "NULL argument");
   DN_TRY(csr_ensure_products(A, r));
   return launch_spmm_t(A, r, W_nr, T_mr);
+}
+
+DN_API int dnpeff_op_spmm_n_variant(dnpeff_csr* A_full, int r, const float* H_mr, float* N_nr,
+                                    int variant) {
+  clear_error();
+  DN_CHECK(A_full && H_mr && N_nr, "NULL argument");
+  DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
+  if (variant == 0) return dnpeff_op_spmm_n(A_full, r, H_mr, N_nr);
+  DN_CHECK(variant == 1 || variant == 2, "variant must be 0 (planned), 1 (a wave per row) or 2 (row chunks)");
+  DN_TRY(csr_ensure_products(A_full, r));
+  dnpeff_csr* A = sparse_part(A_full);
+  DN_CHECK(has_row_major(A), "the row-major arrays of the sparse part were released");
+  DN_TRY(launch_head_n(A_full, r, H_mr));
+  const bool aligned = ((uintptr_t)H_mr % 16) == 0 && ((uintptr_t)N_nr % 16) == 0;
+  if (variant == 1) {
+    if (A->n_rows > 0) {
+      dim3 grid((unsigned)ceil_div(A->n_rows, 4)), block(256);
+      dispatch_gather(r, aligned, [&](auto tag) {
+        using GT = typename decltype(tag)::type;
+        hipLaunchKernelGGL((k_spmm_n_rowwave<GT>), grid, block, 0, stream(), A->rowptr, A->colind,
+                           A->vals, A->n_rows, r, H_mr, N_nr);
+        return 0;
+      });
+      DN_LAUNCH_CHECK();
+    }
+  } else {
+    DN_TRY(csr_ensure_chunks(A));
+    DN_CHECK(A->partials && A->partials_floats >= A->n_chunks * (int64_t)r, "partial sums too small");
+    if (A->n_chunks > 0) {
+      DN_CHECK(A->n_chunks < (int64_t)INT32_MAX, "too many work chunks");
+      dim3 grid((unsigned)A->n_chunks), block(256);
+      const size_t lds = sizeof(float) * 4 * (size_t)r;
+      dispatch_gather(r, ((uintptr_t)H_mr % 16) == 0, [&](auto tag) {
+        using GT = typename decltype(tag)::type;
+        hipLaunchKernelGGL((k_spmm_n<GT>), grid, block, lds, stream(), A->rowptr, A->colind, A->vals,
+                           A->chunk_base, A->n_rows, r, H_mr, A->partials);
+        return 0;
+      });
+      DN_LAUNCH_CHECK();
+    }
+    DN_TRY(launch_chunk_reduce(A, r, A->partials, N_nr));
+  }
+  return launch_head_n_add(A_full, r, N_nr);
 }
 
 DN_API int dnpeff_op_spmm_t_tile(dnpeff_csr* A, int r, const float* W_nr, int64_t col0, int64_t col1,

@@ -36,6 +36,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
@@ -568,8 +569,11 @@ static void spmm_t_f32(const orc_f32_ctx* c, float* out) {
   }
 }
 
-/* G = X^T X, blocked over rows so each thread sums short runs in fp32 and the
- * per-thread blocks are combined in fp64. */
+/* G = X^T X (the cublasSgemm at device_contexts1.h:303,322), register-blocked: eight rows of
+ * X are applied to a row of the local block at a time, so that each element of the block is read
+ * and written once per eight rank-1 updates.  Each thread sums runs of 1024 rows in fp32; the
+ * runs are combined in fp64. */
+#define ORC_RB 8
 static void gram_f32(int64_t rows, int r, const float* X, float* G) {
   double* acc = (double*)calloc((size_t)r * r, sizeof(double));
 #pragma omp parallel
@@ -581,7 +585,22 @@ static void gram_f32(int64_t rows, int r, const float* X, float* G) {
     for (int64_t k0 = 0; k0 < rows; k0 += blk) {
       int64_t k1 = k0 + blk < rows ? k0 + blk : rows;
       for (int i = 0; i < r * r; i++) loc[i] = 0.0f;
-      for (int64_t k = k0; k < k1; k++) {
+      int64_t k = k0;
+      for (; k + ORC_RB <= k1; k += ORC_RB) {
+        const float* x0 = X + k * r;
+        const float *x1 = x0 + r, *x2 = x1 + r, *x3 = x2 + r, *x4 = x3 + r, *x5 = x4 + r,
+                    *x6 = x5 + r, *x7 = x6 + r;
+        for (int a = 0; a < r; a++) {
+          const float a0 = x0[a], a1 = x1[a], a2 = x2[a], a3 = x3[a], a4 = x4[a], a5 = x5[a],
+                      a6 = x6[a], a7 = x7[a];
+          float* l = loc + a * r;
+#pragma omp simd
+          for (int b = 0; b < r; b++)
+            l[b] += ((a0 * x0[b] + a1 * x1[b]) + (a2 * x2[b] + a3 * x3[b])) +
+                    ((a4 * x4[b] + a5 * x5[b]) + (a6 * x6[b] + a7 * x7[b]));
+        }
+      }
+      for (; k < k1; k++) {
         const float* x = X + k * r;
         for (int a = 0; a < r; a++) {
           float xa = x[a];
@@ -601,25 +620,52 @@ static void gram_f32(int64_t rows, int r, const float* X, float* G) {
   free(acc);
 }
 
-/* X <- X * num / (X G + eps), row by row (fused like the device path). */
+/* X <- X * num / (X G + eps) (cublasSgemm + kernelNmfMuUpdate, device_contexts1.h:306-308,
+ * 329-332), eight rows at a time so that a row of G is loaded once per eight rows of X; fused
+ * like the device path. */
 static void xg_mu_f32(int64_t rows, int r, float* X, const float* G, const float* num,
                       float eps) {
 #pragma omp parallel
   {
-    float* d = (float*)malloc(sizeof(float) * r);
+    float* d = (float*)malloc(sizeof(float) * r * ORC_RB);
 #pragma omp for schedule(static)
-    for (int64_t k = 0; k < rows; k++) {
-      float* x = X + k * r;
-      const float* nu = num + k * r;
-      for (int b = 0; b < r; b++) d[b] = 0.0f;
-      for (int a = 0; a < r; a++) {
-        float xa = x[a];
-        const float* g = G + a * r;
+    for (int64_t k0 = 0; k0 < rows; k0 += ORC_RB) {
+      const int nb = rows - k0 < ORC_RB ? (int)(rows - k0) : ORC_RB;
+      for (int i = 0; i < r * ORC_RB; i++) d[i] = 0.0f;
+      if (nb == ORC_RB) {
+        const float* x0 = X + k0 * r;
+        for (int a = 0; a < r; a++) {
+          const float* g = G + a * r;
+          const float a0 = x0[a], a1 = x0[r + a], a2 = x0[2 * r + a], a3 = x0[3 * r + a],
+                      a4 = x0[4 * r + a], a5 = x0[5 * r + a], a6 = x0[6 * r + a], a7 = x0[7 * r + a];
+          float *d0 = d, *d1 = d + r, *d2 = d + 2 * r, *d3 = d + 3 * r, *d4 = d + 4 * r,
+                *d5 = d + 5 * r, *d6 = d + 6 * r, *d7 = d + 7 * r;
 #pragma omp simd
-        for (int b = 0; b < r; b++) d[b] += xa * g[b];
+          for (int b = 0; b < r; b++) {
+            const float gb = g[b];
+            d0[b] += a0 * gb; d1[b] += a1 * gb; d2[b] += a2 * gb; d3[b] += a3 * gb;
+            d4[b] += a4 * gb; d5[b] += a5 * gb; d6[b] += a6 * gb; d7[b] += a7 * gb;
+          }
+        }
+      } else {
+        for (int q = 0; q < nb; q++) {
+          const float* x = X + (k0 + q) * r;
+          float* dq = d + q * r;
+          for (int a = 0; a < r; a++) {
+            const float xa = x[a];
+            const float* g = G + a * r;
+#pragma omp simd
+            for (int b = 0; b < r; b++) dq[b] += xa * g[b];
+          }
+        }
       }
+      for (int q = 0; q < nb; q++) {
+        float* x = X + (k0 + q) * r;
+        const float* nu = num + (k0 + q) * r;
+        const float* dq = d + q * r;
 #pragma omp simd
-      for (int b = 0; b < r; b++) x[b] *= nu[b] / (d[b] + eps);
+        for (int b = 0; b < r; b++) x[b] *= nu[b] / (dq[b] + eps);
+      }
     }
     free(d);
   }
@@ -687,6 +733,63 @@ ORC_API void orc_f32_step(void* ctx, int n_steps) {
     gram_f32(c->n, c->r, c->W, c->G);
     xg_mu_f32(c->m, c->r, c->Ht, c->G, c->num, c->eps);
   }
+}
+
+static double orc_now(void) {
+#ifdef _OPENMP
+  return omp_get_wtime();
+#else
+  return (double)clock() / CLOCKS_PER_SEC;
+#endif
+}
+
+/* The same iteration with the seconds spent in each part added to secs[0..5]:
+ * A H^T, H^T H, W update, A^T W, W^T W, H update. */
+ORC_API void orc_f32_step_timed(void* ctx, int n_steps, double* secs) {
+  orc_f32_ctx* c = (orc_f32_ctx*)ctx;
+  for (int s = 0; s < n_steps; s++) {
+    double t0 = orc_now(), t1;
+    spmm_n_f32(c, c->num);
+    t1 = orc_now(); secs[0] += t1 - t0; t0 = t1;
+    gram_f32(c->m, c->r, c->Ht, c->G);
+    t1 = orc_now(); secs[1] += t1 - t0; t0 = t1;
+    xg_mu_f32(c->n, c->r, c->W, c->G, c->num, c->eps);
+    t1 = orc_now(); secs[2] += t1 - t0; t0 = t1;
+    spmm_t_f32(c, c->num);
+    t1 = orc_now(); secs[3] += t1 - t0; t0 = t1;
+    gram_f32(c->n, c->r, c->W, c->G);
+    t1 = orc_now(); secs[4] += t1 - t0; t0 = t1;
+    xg_mu_f32(c->m, c->r, c->Ht, c->G, c->num, c->eps);
+    t1 = orc_now(); secs[5] += t1 - t0;
+  }
+}
+
+/* fp32 OpenMP port of the first stage of the learner for timing: out[n, r] = A B^T with B given
+ * by its transposed CSR (per column: component ids and values), the product loop of
+ * Partitioned_SpSpMatmul_ToDense (cuda/ops/spsp_matmul.h:95-131).  Returns the seconds taken. */
+ORC_API double orc_f32_spsp_timed(int64_t n, const int64_t* a_rowptr, const int32_t* a_colind,
+                                  const float* a_vals, int r, const int64_t* b_colptr,
+                                  const int32_t* b_comp, const float* b_tvals, float* out_nr) {
+  const double t0 = orc_now();
+#pragma omp parallel for schedule(dynamic, 4)
+  for (int64_t i = 0; i < n; i++) {
+    float* o = out_nr + i * r;
+    for (int c = 0; c < r; c++) o[c] = 0.0f;
+    for (int64_t e = a_rowptr[i]; e < a_rowptr[i + 1]; e++) {
+      const int64_t j = a_colind[e];
+      const float a = a_vals[e];
+      for (int64_t p = b_colptr[j]; p < b_colptr[j + 1]; p++) o[b_comp[p]] += a * b_tvals[p];
+    }
+  }
+  return orc_now() - t0;
+}
+
+/* fp32 port of the learner's second stage for timing: n_steps of W <- W * AH / (W HH + eps). */
+ORC_API double orc_f32_fit_steps_timed(int64_t n, int r, const float* AH, const float* HH, float eps,
+                                       int n_steps, float* W) {
+  const double t0 = orc_now();
+  for (int s = 0; s < n_steps; s++) xg_mu_f32(n, r, W, HH, AH, eps);
+  return orc_now() - t0;
 }
 
 ORC_API void orc_f32_get(void* ctx, float* W, float* H_rm) {

@@ -56,6 +56,9 @@ _fit = _sig(_lib, "orc_fit_f64", None, [_i64, C.c_int, _p, _p, _f64, _f32, C.c_i
 _f32_create = _sig(_lib, "orc_f32_create", _p, [_i64, _i64, _p, _p, _p, C.c_int, _f32, _p, _p])
 _f32_create_mr = _sig(_lib, "orc_f32_create_mr", _p, [_i64, _i64, _p, _p, _p, C.c_int, _f32, _p, _p])
 _f32_step = _sig(_lib, "orc_f32_step", None, [_p, C.c_int])
+_f32_step_timed = _sig(_lib, "orc_f32_step_timed", None, [_p, C.c_int, _p])
+_f32_spsp_timed = _sig(_lib, "orc_f32_spsp_timed", _f64, [_i64, _p, _p, _p, C.c_int, _p, _p, _p, _p])
+_f32_fit_timed = _sig(_lib, "orc_f32_fit_steps_timed", _f64, [_i64, C.c_int, _p, _p, _f32, C.c_int, _p])
 _f32_get = _sig(_lib, "orc_f32_get", None, [_p, _p, _p])
 _f32_destroy = _sig(_lib, "orc_f32_destroy", None, [_p])
 _num_threads = _sig(_lib, "orc_num_threads", C.c_int, [])
@@ -245,6 +248,14 @@ class F32Baseline:
     def step(self, n_steps=1):
         _f32_step(self._h, n_steps)
 
+    PARTS = ("spmm_n", "gram_H", "xg_mu_W", "spmm_t", "gram_W", "xg_mu_H")
+
+    def step_timed(self, n_steps=1):
+        """Seconds spent in each part of n_steps iterations, keyed like the device kernel classes."""
+        secs = np.zeros(6, dtype=np.float64)
+        _f32_step_timed(self._h, n_steps, _ptr(secs))
+        return dict(zip(self.PARTS, secs.tolist()))
+
     def get(self):
         W = np.zeros((self.n, self.r), dtype=np.float32)
         H = np.zeros((self.r, self.m), dtype=np.float32)
@@ -259,6 +270,27 @@ class F32Baseline:
     @staticmethod
     def num_threads():
         return _num_threads()
+
+
+def spsp_f32_timed(a_csr, b_transposed, r):
+    """fp32 OpenMP A B^T (first stage of the learner) on the host cores: (out [n, r], seconds).
+    b_transposed = (colptr, component ids, values) of B's transposed CSR."""
+    ar, ac, av = _csr(*a_csr)
+    bp, bc, bv = _csr(*b_transposed)
+    n = len(ar) - 1
+    out = np.zeros((n, r), dtype=np.float32)
+    secs = _f32_spsp_timed(n, _ptr(ar), _ptr(ac), _ptr(av), r, _ptr(bp), _ptr(bc), _ptr(bv), _ptr(out))
+    return out, secs
+
+
+def fit_steps_f32_timed(AH, HH, W0, eps, n_steps):
+    """n_steps of the learner's W update in fp32 on the host cores: (W, seconds)."""
+    AH = np.ascontiguousarray(AH, dtype=np.float32)
+    HH = np.ascontiguousarray(HH, dtype=np.float32)
+    W = np.array(W0, dtype=np.float32, copy=True, order="C")
+    n, r = W.shape
+    secs = _f32_fit_timed(n, r, _ptr(AH), _ptr(HH), eps, n_steps, _ptr(W))
+    return W, secs
 
 
 # ---- compiled reference routines (oracle/_ref) ----------------------------------------------

@@ -139,6 +139,35 @@ def test_f32_baseline_tracks_f64_oracle():
     assert np.linalg.norm(H32 - H64) / np.linalg.norm(H64) < 1e-5
 
 
+def test_f32_timed_parts_run_the_same_iteration_and_fit_parts_match_f64():
+    """The timed variants used by bench.py's cpu_baseline compute what the untimed ones do (the
+    timing must not be of a different loop), the fp32 first-stage product and W update of the
+    learner agree with the fp64 restatement."""
+    rng = np.random.default_rng(23)
+    n, m, r = 37, 411, 19  # neither a multiple of the 8-row blocks
+    rp, ci, va = random_csr(rng, n, m, 90)
+    W0, H0 = rng.random((n, r)).astype(np.float32), rng.random((r, m)).astype(np.float32)
+    a = orc.F32Baseline(rp, ci, va, m, W0, H0, np.float32(1e-8))
+    b = orc.F32Baseline(rp, ci, va, m, W0, H0, np.float32(1e-8))
+    a.step(3)
+    parts = b.step_timed(3)
+    assert set(parts) == set(orc.F32Baseline.PARTS) and all(v >= 0 for v in parts.values())
+    for x, y in zip(a.get(), b.get()):
+        assert np.array_equal(x, y)
+    a.close()
+    b.close()
+    # learner: A B^T with sparse B, then W updates
+    brp, bci, bva = random_csr(rng, r, m, 60, sort_cols=True)
+    bt = orc.transpose(brp, bci, bva, m)
+    out32, secs = orc.spsp_f32_timed((rp, ci, va), bt, r)
+    out64 = orc.spsp_dense_f64((rp, ci, va), m, (brp, bci, bva), r)
+    assert secs >= 0 and np.allclose(out32, out64, rtol=1e-5, atol=1e-7)
+    HH = orc.spsp_dense_f64((brp, bci, bva), m, (brp, bci, bva), r)
+    W32, secs = orc.fit_steps_f32_timed(out64, HH, W0, np.float32(1e-7), 4)
+    W64, _, _ = orc.fit_f64(out64, HH, 1.0, W0, np.float32(1e-7), 4, log_every=0)
+    assert np.linalg.norm(W32 - W64) / np.linalg.norm(W64) < 1e-5
+
+
 def test_sparsify_H_keeps_the_product_and_thresholds_unit_norm_rows():
     """The product W H is unchanged by the normalisation, kept rows have unit norm, threshold 0
     on non-negative H keeps every entry, and a dense rebuild of the CSR equals the thresholded
