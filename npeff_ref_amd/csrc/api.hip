@@ -165,7 +165,7 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
   double avail = (double)free_b;
   if (consume && A->colind && A->vals) avail += 8.0 * (double)A->nnz;
   if (A->tail) {
-    avail += 8.0 * (double)A->head.n_pad * (double)A->head.n_d_pad;
+    avail += (A->head.rm ? 8.0 : 4.0) * (double)A->head.n_pad * (double)A->head.n_d_pad;
     if (S0->colind) avail += 8.0 * (double)S0->nnz;
   }
   if (S0->colptr) avail += 8.0 * (double)S0->nnz;
@@ -179,7 +179,8 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
   *tiled = tn.tiled_h > 0.0;
   if (A->tail) {
     if (rank % 4 == 0) {  // split by the caller (or an earlier handle): keep it
-      const double foot = 8.0 * (double)A->head.n_pad * (double)A->head.n_d_pad + 16.0 * (double)S0->nnz;
+      const double foot = 4.0 * head_blocks_for_rank(rank) * (double)A->head.n_pad * (double)A->head.n_d_pad +
+                          16.0 * (double)S0->nnz;
       if (tn.tiled_h < 0.0) *tiled = foot > budget_full;
       return 0;
     }
@@ -192,10 +193,11 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
     return 0;
   }
   head_choice c;
-  DN_TRY(choose_dense_head(A, fill, *tiled ? budget_tiled : budget_full, &c));
+  const int n_blocks = head_blocks_for_rank(rank);
+  DN_TRY(choose_dense_head(A, fill, *tiled ? budget_tiled : budget_full, n_blocks, &c));
   if (!c.fits && tn.tiled_h < 0.0 && !*tiled) {
     *tiled = true;
-    DN_TRY(choose_dense_head(A, fill, budget_tiled, &c));
+    DN_TRY(choose_dense_head(A, fill, budget_tiled, n_blocks, &c));
   }
   if (tn.verbose != 0.0)
     fprintf(stderr,

@@ -174,7 +174,9 @@ struct dense_head {
   int64_t n_pad = 0;    // rows rounded up to 128
   int32_t* cols = nullptr;  // [n_d] column of each head slot, ascending
   float* cm = nullptr;      // [n_d_pad, n_pad]: cm[k * n_pad + i] = A[i, cols[k]]
-  float* rm = nullptr;      // [n_pad, n_d_pad]: rm[i * n_d_pad + k] = A[i, cols[k]]
+  // [n_pad, n_d_pad]: rm[i * n_d_pad + k] = A[i, cols[k]]; made from cm when a product needs it
+  // (the fp32 matrix-core kernel of A^T W; the split-operand kernels read cm in both directions)
+  float* rm = nullptr;
   float* ws = nullptr;      // gathered factor rows + slice partials of the products
   int64_t ws_floats = 0;
 };
@@ -282,7 +284,9 @@ struct head_choice {
   bool fits = true;        // footprint within the budget given
 };
 constexpr double NO_BUDGET = 1e300;
-int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, head_choice* out);
+int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_blocks, head_choice* out);
+// Dense blocks that the head's products at rank r read (1 or 2), see dense_head::rm.
+int head_blocks_for_rank(int r);
 int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense);
 // Frees every array of A that the products A H^T and A^T W do not read.
 int csr_consume_for_products(dnpeff_csr* A);

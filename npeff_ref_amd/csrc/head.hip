@@ -1,5 +1,6 @@
 // Dense head of a sparse matrix: the columns that are present in a sizeable fraction of the
-// rows are taken out of the CSR structures and kept as a dense block, in both orientations.
+// rows are taken out of the CSR structures and kept as a dense block ("cm", one head column after
+// the other; a second copy "rm" in the other orientation only for the fp32 kernel of A^T W).
 // Their share of A H^T and A^T W is then a matrix product on fp32 MFMA (32x32x2) instead of one
 // 4r-byte gather per entry; the remaining ("tail") entries stay sparse.
 //
@@ -216,6 +217,8 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
 // Operands are zero-padded to whole tiles (rows to M_pad / N, the contraction to a multiple of
 // 32 within lda / ldb), so the loads need no bounds.
 // ---------------------------------------------------------------------------
+// A_KN: A is stored with the contraction index slow (A[k * lda + row], lda >= M_pad).
+template <bool A_KN>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_abt_b16(const float* __restrict__ A, int64_t lda, const float* __restrict__ B, int64_t ldb,
               int64_t K, int N, int64_t M, int64_t M_pad, float* __restrict__ out) {
@@ -236,7 +239,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-  abt_mainloop<false, false>(A + m0 * lda, lda, B + (int64_t)n0 * ldb, ldb, z, S, n_my, ab, acc);
+  abt_mainloop<A_KN, false>(A_KN ? A + m0 : A + m0 * lda, lda, B + (int64_t)n0 * ldb, ldb, z, S, n_my, ab,
+                            acc);
 
   // D layout of a 32x32 block: reg v of lane l holds row 8 (v/4) + 4 (l/32) + v%4, column l%32;
   // block (i, j) of the wave covers rows 64 wm + 32 i.., columns 64 wn + 32 j.. of the tile.
@@ -253,20 +257,26 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 static int launch_abt_b16(const float* A, int64_t lda, const float* B, int64_t ldb, int64_t K, int N,
-                          int64_t M, int64_t M_pad, int64_t slices, float* out) {
+                          int64_t M, int64_t M_pad, int64_t slices, float* out, bool a_kn = false) {
   static bool attr_set = false;
   if (!attr_set) {
-    DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_abt_b16),
+    DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_abt_b16<false>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+    DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_abt_b16<true>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
     attr_set = true;
   }
   const int64_t k_pad = ceil_div(K, ABT_KB) * ABT_KB;
-  DN_CHECK(M_pad % 128 == 0 && N % 128 == 0 && lda % 4 == 0 && ldb % 4 == 0 && k_pad <= lda &&
-               k_pad <= ldb && ((uintptr_t)A % 16) == 0 && ((uintptr_t)B % 16) == 0,
+  DN_CHECK(M_pad % 128 == 0 && N % 128 == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
+               (a_kn ? M_pad <= lda : k_pad <= lda) && k_pad <= ldb && ((uintptr_t)A % 16) == 0 &&
+               ((uintptr_t)B % 16) == 0,
            "dense product: misaligned or unpadded operands");
   DN_CHECK(M_pad / 128 < ((int64_t)1 << 22), "dense product: too many row tiles");
   dim3 grid((unsigned)(M_pad / 128), (unsigned)(N / 128), (unsigned)slices);
-  hipLaunchKernelGGL(k_abt_b16, grid, dim3(256), ABT_LDS, stream(), A, lda, B, ldb, K, N, M, M_pad, out);
+  if (a_kn)
+    hipLaunchKernelGGL(k_abt_b16<true>, grid, dim3(256), ABT_LDS, stream(), A, lda, B, ldb, K, N, M, M_pad, out);
+  else
+    hipLaunchKernelGGL(k_abt_b16<false>, grid, dim3(256), ABT_LDS, stream(), A, lda, B, ldb, K, N, M, M_pad, out);
   DN_LAUNCH_CHECK();
   return 0;
 }
@@ -488,6 +498,7 @@ static unsigned elem_grid(int64_t count) {
 // At ranks that are multiples of 128 the head products run on the bf16 matrix cores with split
 // operands (k_abt_b16), otherwise (and with DNPEFF_SPLIT_BF16=0) on the fp32 ones (k_ptq).
 static bool head_uses_split(int r) { return r % 128 == 0 && use_split_bf16(); }
+int head_blocks_for_rank(int r) { return head_uses_split(r) ? 1 : 2; }
 static int64_t head_gather_floats(const dense_head& h, int r) {
   return (h.n_d_pad > h.n_pad ? h.n_d_pad : h.n_pad) * (int64_t)r;
 }
@@ -509,6 +520,10 @@ int head_ensure_workspace(dnpeff_csr* A, int r) {
   const int64_t wn = head_slices_n(h, r) * h.n_pad * r;
   const int64_t wt = head_slices_t(h, r, A->n_rows) * h.n_d_pad * r;
   const int64_t need = gather + (wn > wt ? wn : wt);
+  if (!head_uses_split(r) && !h.rm) {  // the fp32 kernel of A^T W wants the block row by row
+    DN_TRY(dmalloc(&h.rm, h.n_pad * h.n_d_pad));
+    DN_TRY(launch_transpose(h.n_d_pad, h.n_pad, h.cm, h.rm));
+  }
   if (h.ws && h.ws_floats >= need) return 0;
   dfree(h.ws);
   h.ws = nullptr;
@@ -525,11 +540,12 @@ int launch_head_n(const dnpeff_csr* A, int r, const float* H_mr) {
   float* Hd = h.ws;
   float* part = h.ws + head_gather_floats(h, r);
   if (head_uses_split(r)) {
-    // D [n, n_d] (rm) times the gathered rows, transposed: contraction over the head slots
+    // D [n, n_d] (cm, read with the contraction index slow) times the gathered rows, transposed:
+    // contraction over the head slots
     dim3 tg((unsigned)ceil_div(h.n_d_pad, 32), (unsigned)ceil_div(r, 32));
     hipLaunchKernelGGL(k_head_gather_t, tg, dim3(256), 0, stream(), H_mr, h.cols, h.n_d, r, h.n_d_pad, Hd);
-    return launch_abt_b16(h.rm, h.n_d_pad, Hd, h.n_d_pad, h.n_d, r, A->n_rows, h.n_pad,
-                          head_slices_n(h, r), part);
+    return launch_abt_b16(h.cm, h.n_pad, Hd, h.n_d_pad, h.n_d, r, A->n_rows, h.n_pad,
+                          head_slices_n(h, r), part, /*a_kn=*/true);
   }
   hipLaunchKernelGGL(k_head_gather, dim3(elem_grid(h.n_d * (r / 4))), dim3(256), 0, stream(), H_mr,
                      h.cols, h.n_d, r, Hd);
@@ -561,6 +577,7 @@ int launch_head_t_product(const dnpeff_csr* A, int r, const float* W_nr) {
     hipLaunchKernelGGL(k_transpose_pad, tg, dim3(256), 0, stream(), W_nr, A->n_rows, r, h.n_pad, Wt);
     return launch_abt_b16(h.cm, h.n_pad, Wt, h.n_pad, A->n_rows, r, h.n_d, h.n_d_pad, slices, part);
   }
+  DN_CHECK(h.rm != nullptr, "dense head: no row-major block for the fp32 product");
   return launch_ptq(h.rm, h.n_d_pad, A->n_rows, W_nr, r, h.n_d, h.n_d_pad, slices, part);
 }
 

@@ -184,20 +184,17 @@ __global__ void __launch_bounds__(256)
     table[i] = og_to_new[i] >= 0 ? -1 : (int32_t)i;
 }
 
-// Entries of the head's columns into both dense blocks; a workgroup per row.  Entries that
-// repeat a (row, column) pair add up, as they do in the sparse products.
+// Entries of the head's columns into the dense block; a workgroup per row.  (A matrix whose rows
+// hold a column twice is refused by the products, so every element receives one addition.)
 __global__ void __launch_bounds__(256)
     k_head_fill(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
                 const float* __restrict__ vals, int64_t n_rows, const int32_t* __restrict__ slot_of,
-                float* __restrict__ cm, int64_t n_pad, float* __restrict__ rm, int64_t n_d_pad) {
+                float* __restrict__ cm, int64_t n_pad) {
   for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
     const int64_t e1 = rowptr[row + 1];
     for (int64_t e = rowptr[row] + threadIdx.x; e < e1; e += 256) {
       const int32_t k = slot_of[colind[e]];
-      if (k >= 0) {
-        atomicAdd(&cm[(int64_t)k * n_pad + row], vals[e]);
-        atomicAdd(&rm[row * n_d_pad + k], vals[e]);
-      }
+      if (k >= 0) atomicAdd(&cm[(int64_t)k * n_pad + row], vals[e]);
     }
   }
 }
@@ -1097,12 +1094,13 @@ __global__ void __launch_bounds__(256)
 namespace dn {
 
 // Which columns form the dense head.  Candidates are the thresholds thr0, 2 thr0, 4 thr0, ...
-// (thr0 = ceil(min_fill n_rows)) and "no head"; a candidate is admissible when both dense blocks
-// stay below an eighth of the device memory; its footprint is the two blocks plus both sparse
-// copies of the remaining entries (16 bytes each).  The choice is the first admissible candidate
+// (thr0 = ceil(min_fill n_rows)) and "no head"; a candidate is admissible when its dense blocks
+// (n_blocks of them: one where the products read it in both directions, two otherwise) stay
+// below a sixth of the device memory; its footprint is the blocks plus both sparse copies of
+// the remaining entries (16 bytes each).  The choice is the first admissible candidate
 // whose footprint is within `budget` bytes (NO_BUDGET: the first admissible one), else the
 // admissible candidate with the smallest footprint (fits = false).
-int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, head_choice* out) {
+int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_blocks, head_choice* out) {
   *out = head_choice();
   out->footprint = 16.0 * (double)A->nnz;
   out->fits = out->footprint <= budget;
@@ -1138,8 +1136,8 @@ int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, head_choice
                        zsum.p);
     DN_LAUNCH_CHECK();
     DN_HIP(hipMemcpy(&z_head, zsum, sizeof(unsigned long long), hipMemcpyDeviceToHost));
-    const double blocks = 2.0 * 4.0 * (double)n_pad * (double)(ceil_div(n_d, 128) * 128);
-    if (blocks > (double)total_b / 8.0) continue;
+    const double blocks = n_blocks * 4.0 * (double)n_pad * (double)(ceil_div(n_d, 128) * 128);
+    if (blocks > (double)total_b / 6.0) continue;
     head_choice c;
     c.thr = thr;
     c.n_d = n_d;
@@ -1188,13 +1186,11 @@ int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense) {
   DN_HIP(hipStreamSynchronize(st));
   count.reset();
   pos.reset();
-  dbuf<float> cm, rm;
+  dbuf<float> cm;
   DN_TRY(cm.alloc(n_d_pad * n_pad));
-  DN_TRY(rm.alloc(n_pad * n_d_pad));
   DN_HIP(hipMemsetAsync(cm, 0, sizeof(float) * (size_t)(n_d_pad * n_pad), st));
-  DN_HIP(hipMemsetAsync(rm, 0, sizeof(float) * (size_t)(n_pad * n_d_pad), st));
   hipLaunchKernelGGL(k_head_fill, dim3(grid_for(n * 256)), dim3(256), 0, st, A->rowptr, A->colind,
-                     A->vals, n, slot_of.p, cm.p, n_pad, rm.p, n_d_pad);
+                     A->vals, n, slot_of.p, cm.p, n_pad);
   DN_LAUNCH_CHECK();
   // the remaining entries: the row-major arrays without the head's columns, written straight
   // into the tail's own arrays (positions from a scan over the entries)
@@ -1227,7 +1223,7 @@ int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense) {
   }
   dense_head& h = A->head;
   h.n_d = n_d; h.n_d_pad = n_d_pad; h.n_pad = n_pad;
-  h.cols = cols.release(); h.cm = cm.release(); h.rm = rm.release();
+  h.cols = cols.release(); h.cm = cm.release();
   A->tail = T;
   if (n_dense) *n_dense = n_d;
   return 0;
@@ -1245,7 +1241,7 @@ DN_API int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* 
     return 0;
   }
   head_choice c;
-  DN_TRY(choose_dense_head(A, min_fill, NO_BUDGET, &c));
+  DN_TRY(choose_dense_head(A, min_fill, NO_BUDGET, 2, &c));
   return split_dense_head_at(A, c.thr, n_dense);
 }
 
@@ -1404,8 +1400,8 @@ DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* 
   if (A->head.n_d) {
     head_row.resize((size_t)A->head.n_d);
     head_cols.resize((size_t)A->head.n_d);
-    DN_HIP(hipMemcpy(head_row.data(), A->head.rm + row * A->head.n_d_pad, sizeof(float) * A->head.n_d,
-                     hipMemcpyDeviceToHost));
+    DN_HIP(hipMemcpy2D(head_row.data(), sizeof(float), A->head.cm + row, sizeof(float) * A->head.n_pad,
+                       sizeof(float), (size_t)A->head.n_d, hipMemcpyDeviceToHost));
     DN_HIP(hipMemcpy(head_cols.data(), A->head.cols, sizeof(int32_t) * A->head.n_d,
                      hipMemcpyDeviceToHost));
     for (float v : head_row) got += v != 0.0f;
