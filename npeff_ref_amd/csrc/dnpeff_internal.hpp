@@ -153,10 +153,10 @@ struct tuning_t {
   double sweep_waves = 0.0;        // waves per workgroup of the sweep kernel (0 = as many as fit)
   double sweep_lag = 0.0;          // pieces the workgroups of an XCD may be apart
   double sweep_spin = 400.0;       // polls before a workgroup of the sweep stops waiting
-  double spmm_t_slices = 1.0;      // component slices of A^T W
+  double spmm_t_slices = 0.0;      // component slices of A^T W (0 = by the size of W)
   double split_bf16 = 1.0;         // matrix products on the bf16 cores with split fp32 operands (0 = fp32 cores)
   double fused_gram = 1.0;         // rank 128: the H update also produces H^T H
-  double h_tile_mb = 128.0;        // size of a column tile of the tiled H update, MiB of the factor
+  double h_tile_mb = 768.0;        // size of a column tile of the tiled H update, MiB of the factor
   double tiled_h = -1.0;           // tiled H update: 1 = always, 0 = never, -1 = when the full-size buffer does not fit
   double topk_fast_cap = -1.0;     // top-k: candidate list length that ends the histogram passes (-1 = default)
   double verbose = 0.0;

@@ -669,13 +669,18 @@ constexpr int SPMM_T_COLS = 32;
 template <int LPR, int T, bool FULL, bool SMALL>
 __global__ void __launch_bounds__(256)
     k_spmm_t_grouped(const int64_t* __restrict__ colptr, const int32_t* __restrict__ rowind,
-                     const float* __restrict__ tvals, int64_t m, int r,
+                     const float* __restrict__ tvals, int64_t m, int r, int n_slices,
                      const float* __restrict__ W, float* __restrict__ Tout) {
   constexpr int G = 64 / LPR;
   constexpr int UNR = T >= 4 ? 1 : T == 2 ? 2 : 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int sub = lane % LPR, grp = lane / LPR, gbase = grp * LPR;
-  const int64_t j0 = ((int64_t)blockIdx.x * 4 + wave) * SPMM_T_COLS;
+  // With component slices, workgroup b works on slice b % n_slices (4 LPR T components starting
+  // at that multiple): the XCD it runs on gathers from its own slice of W only.
+  const int slice = blockIdx.x % n_slices;
+  W += slice * (4 * LPR * T);
+  Tout += slice * (4 * LPR * T);
+  const int64_t j0 = ((int64_t)(blockIdx.x / n_slices) * 4 + wave) * SPMM_T_COLS;
   if (j0 >= m) return;
   bool ok[T];
 #pragma unroll
@@ -1125,14 +1130,20 @@ int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float
   return 0;
 }
 
-// Component slices for A^T W.  Measured on configs[1] (n = 10,000, r = 128): 1 slice 29 ms,
-// 2 slices 37 ms, 4 slices 64 ms -- re-reading the entries once per slice costs more than the
-// better L2 residency of W gains, so the default is 1.  The spmm_t_slices switch (2, 4 or 8)
-// selects a sliced launch (for experiments on other shapes).
-static int spmm_t_slices(int64_t /*n*/, int r) {
-  const int v = (int)tuning().spmm_t_slices;
-  if ((v == 2 || v == 4 || v == 8) && r % v == 0 && (r / v) % 4 == 0) return v;
-  return 1;
+// Component slices for A^T W: workgroup b gathers slice b % n_slices of the rows of W, so an XCD
+// (workgroups are dealt to the XCDs round-robin) only ever touches its own slice and keeps more
+// of it in its 4 MB L2, at the price of reading the entries once per slice.  Measured with the
+// grouped kernel, 1 / 2 / 4 / 8 slices: 10,000 x 128 (W 5.1 MB) 19.6 / 19.0 / 20.7 / 40.5 ms,
+// 20,000 x 256 (W 20.5 MB) 352 / 294 / 230 / 246 ms.  Rule: the fewest slices (1, 2, 4, 8) that
+// bring a slice of W to 6 MB or less, slices of at least 16 components; the spmm_t_slices
+// switch overrides it (0 = this rule).
+static int spmm_t_slices(int64_t n, int r) {
+  auto ok = [&](int v) { return r % v == 0 && (r / v) % 16 == 0; };
+  const int forced = (int)tuning().spmm_t_slices;
+  if (forced == 1 || ((forced == 2 || forced == 4 || forced == 8) && ok(forced))) return forced;
+  int v = 1;
+  while (v < 8 && ok(2 * v) && 4.0 * (double)n * r / v > 6.0e6) v *= 2;
+  return v;
 }
 
 // The sparse part of rows [col0, col1) of A^T W into T (row j - col0); long_cols[l0 .. l1) are the
@@ -1152,29 +1163,31 @@ static int launch_spmm_t_sparse(const dnpeff_csr* A, int r, const float* W_nr, f
   const int64_t max_wgs = ((int64_t)1 << 23) / n_slices * n_slices;
   if (wgs > max_wgs) wgs = max_wgs;
   dim3 grid((unsigned)wgs), block(256);
-  const bool grouped = aligned && r % 4 == 0 && n_slices == 1;
+  // the grouped kernel handles whole slices of 16, 32, ..., 256 components (or the whole rank)
+  const bool slice_ok = n_slices == 1 || width == 16 || width == 32 || width == 64 || width == 128 || width == 256;
+  const bool grouped = aligned && r % 4 == 0 && slice_ok;
   const bool w_small = (double)A->n_rows * r * 4.0 < 4.0e9;  // 32-bit offsets into W
   if (grouped) {
-    dim3 gg((unsigned)ceil_div(m, 4 * SPMM_T_COLS));
-    const int r4 = r / 4;
+    dim3 gg((unsigned)(ceil_div(m, 4 * SPMM_T_COLS) * n_slices));
+    const int w4 = width / 4;
 #define DN_GROUPED2(LPR, T_, FULL, SMALL)                                                     \
   hipLaunchKernelGGL((k_spmm_t_grouped<LPR, T_, FULL, SMALL>), gg, block, 0, stream(), colptr, \
-                     A->rowind, A->tvals, m, r, W_nr, T)
+                     A->rowind, A->tvals, m, r, n_slices, W_nr, T)
 #define DN_GROUPED(LPR, T_)                                     \
   do {                                                          \
-    const bool full = r == 4 * LPR * T_;                        \
+    const bool full = width == 4 * LPR * T_;                    \
     if (full && w_small24) DN_GROUPED2(LPR, T_, true, true);    \
     else if (full) DN_GROUPED2(LPR, T_, true, false);           \
     else if (w_small24) DN_GROUPED2(LPR, T_, false, true);      \
     else DN_GROUPED2(LPR, T_, false, false);                    \
   } while (0)
     const bool w_small24 = w_small && A->n_rows < ((int64_t)1 << 24);
-    if (r4 <= 4) DN_GROUPED(4, 1);
-    else if (r4 <= 8) DN_GROUPED(8, 1);
-    else if (r4 <= 16) DN_GROUPED(16, 1);
-    else if (r4 <= 32) DN_GROUPED(32, 1);
-    else if (r4 <= 64) DN_GROUPED(64, 1);
-    else if (r4 <= 128) DN_GROUPED(64, 2);
+    if (w4 <= 4) DN_GROUPED(4, 1);
+    else if (w4 <= 8) DN_GROUPED(8, 1);
+    else if (w4 <= 16) DN_GROUPED(16, 1);
+    else if (w4 <= 32) DN_GROUPED(32, 1);
+    else if (w4 <= 64) DN_GROUPED(64, 1);
+    else if (w4 <= 128) DN_GROUPED(64, 2);
     else DN_GROUPED(64, 4);
 #undef DN_GROUPED2
 #undef DN_GROUPED

@@ -28,11 +28,15 @@ __global__ void __launch_bounds__(256)
   if (i < n_rows) len[i] = (int)dn_row_length(seed, (uint64_t)i, k_fixed, k_min, k_max);
 }
 
-// One workgroup draws one row at a time.  Batches of 256 draws (draw index t =
-// batch base + thread id) are inserted into a per-workgroup open-addressing
-// table keyed by id holding the smallest draw index seen; a draw is accepted
-// iff it is the first occurrence of its id, and accepted draws are written in
-// draw order.  This reproduces sequential sampling with rejection exactly.
+// One workgroup draws one row at a time.  Batches of 256 SYNTH_D draws (thread tid holds the
+// draws batch base + SYNTH_D tid + q, q < SYNTH_D) are inserted into a per-workgroup
+// open-addressing table keyed by id holding the smallest draw index seen; a draw is accepted iff
+// it is the first occurrence of its id, and accepted draws are written in draw order.  This
+// reproduces sequential sampling with rejection exactly.  Most draws of a skewed distribution
+// repeat an id that an earlier batch has put into the table: such a draw sees the id with a
+// smaller draw index on a plain read and needs no atomic operation.
+constexpr int SYNTH_D = 8;
+
 __global__ void __launch_bounds__(256)
     k_synth_cols(dn_zipf z, uint64_t seed, int64_t n_rows, const int64_t* __restrict__ rowptr,
                  int32_t* __restrict__ colind, unsigned long long* table_all, uint64_t cap,
@@ -51,33 +55,51 @@ __global__ void __launch_bounds__(256)
 
     int64_t count = 0;
     const uint64_t budget = draw_budget(k);
-    for (uint64_t t_base = 0; count < k && t_base < budget; t_base += 256) {
-      const uint64_t t = t_base + tid;
-      const uint64_t id = (uint64_t)dn_zipf_draw(&z, seed, (uint64_t)row, t);
-      const unsigned long long packed = (id << 32) | t;
-      uint64_t slot = slot_hash(id) & mask;
-      for (;;) {
-        unsigned long long old = atomicCAS(&table[slot], SLOT_EMPTY, packed);
-        if (old == SLOT_EMPTY) break;
-        if ((old >> 32) == id) {
-          atomicMin(&table[slot], packed);
-          break;
+    for (uint64_t t_base = 0; count < k && t_base < budget; t_base += 256 * SYNTH_D) {
+      uint64_t ids[SYNTH_D], slots[SYNTH_D];
+      bool maybe[SYNTH_D];  // not yet known to repeat an earlier draw
+#pragma unroll
+      for (int q = 0; q < SYNTH_D; q++) {
+        const uint64_t t = t_base + (uint64_t)tid * SYNTH_D + q;
+        const uint64_t id = (uint64_t)dn_zipf_draw(&z, seed, (uint64_t)row, t);
+        const unsigned long long packed = (id << 32) | t;
+        uint64_t slot = slot_hash(id) & mask;
+        bool open = true;
+        for (;;) {
+          unsigned long long cur = __hip_atomic_load(&table[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (cur == SLOT_EMPTY) {
+            cur = atomicCAS(&table[slot], SLOT_EMPTY, packed);
+            if (cur == SLOT_EMPTY) break;
+          }
+          if ((cur >> 32) == id) {
+            if ((cur & 0xffffffffULL) < t) open = false;  // an earlier draw holds the id
+            else atomicMin(&table[slot], packed);
+            break;
+          }
+          slot = (slot + 1) & mask;
         }
-        slot = (slot + 1) & mask;
+        ids[q] = id;
+        slots[q] = slot;
+        maybe[q] = open;
       }
       __threadfence();
       __syncthreads();
-      // first occurrence of this id?
-      slot = slot_hash(id) & mask;
-      unsigned long long cur;
-      for (;;) {
-        cur = __hip_atomic_load(&table[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((cur >> 32) == id) break;
-        slot = (slot + 1) & mask;
+      // first occurrence of its id?  (the slot of an id never moves)
+      int wins = 0;
+      bool win[SYNTH_D];
+#pragma unroll
+      for (int q = 0; q < SYNTH_D; q++) {
+        win[q] = false;
+        if (maybe[q]) {
+          const uint64_t t = t_base + (uint64_t)tid * SYNTH_D + q;
+          const unsigned long long cur =
+              __hip_atomic_load(&table[slots[q]], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          win[q] = (cur & 0xffffffffULL) == t;
+        }
+        wins += win[q] ? 1 : 0;
       }
-      const int win = ((cur & 0xffffffffULL) == t) ? 1 : 0;
-      // exclusive scan of win over the workgroup, in draw order
-      sh[tid] = win;
+      // exclusive scan of the per-thread counts over the workgroup, in draw order
+      sh[tid] = wins;
       __syncthreads();
       for (int off = 1; off < 256; off <<= 1) {
         int add = tid >= off ? sh[tid - off] : 0;
@@ -88,8 +110,13 @@ __global__ void __launch_bounds__(256)
       const int incl = sh[tid];
       const int total = sh[255];
       __syncthreads();
-      const int64_t pos = count + incl - win;
-      if (win && pos < k) colind[base + pos] = (int32_t)id;
+      int64_t pos = count + incl - wins;
+#pragma unroll
+      for (int q = 0; q < SYNTH_D; q++)
+        if (win[q]) {
+          if (pos < k) colind[base + pos] = (int32_t)ids[q];
+          pos++;
+        }
       count += total;
     }
     if (count < k && tid == 0) atomicAdd(failed, 1);
@@ -174,7 +201,10 @@ DN_API int dnpeff_synth_pef(int64_t n_rows, int64_t n_cols, int64_t k_fixed, int
   const int64_t kmax_eff = k_min > 0 ? k_max : k_fixed;
   uint64_t cap = 1024;
   while (cap < 2 * (uint64_t)(kmax_eff + 256)) cap <<= 1;
-  int64_t wgs = 2 * (int64_t)n_cus();
+  // the draws are long chains of fp64 arithmetic: as many workgroups as the tables leave room for
+  // (one table each, at most 24 GB together), up to 8 per CU
+  int64_t wgs = 8 * (int64_t)n_cus();
+  while (wgs > 2 * (int64_t)n_cus() && (double)wgs * (double)cap * 8.0 > 24e9) wgs /= 2;
   if (wgs > n_rows) wgs = n_rows;
   if (wgs < 1) wgs = 1;
   if (dmalloc(&tables, (int64_t)(cap * (uint64_t)wgs))) return fail(1);
