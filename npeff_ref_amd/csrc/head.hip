@@ -503,11 +503,20 @@ static int64_t head_gather_floats(const dense_head& h, int r) {
   return (h.n_d_pad > h.n_pad ? h.n_d_pad : h.n_pad) * (int64_t)r;
 }
 
+// Slices of the contraction: enough workgroups to fill the chip, and no fp32 running sum longer
+// than 8192 products (the slices are added in fp64).
+static int64_t head_slices_for(int64_t tiles_mn, int64_t K) {
+  const int64_t k_tiles = ceil_div(K, PTQ_KB);
+  int64_t s = ptq_slices(tiles_mn, k_tiles);
+  const int64_t by_length = ceil_div(K, 8192);
+  if (s < by_length) s = by_length;
+  return s < k_tiles ? s : (k_tiles > 0 ? k_tiles : 1);
+}
 static int64_t head_slices_n(const dense_head& h, int r) {
-  return ptq_slices((h.n_pad / 128) * ceil_div(r, 128), ceil_div(h.n_d, PTQ_KB));
+  return head_slices_for((h.n_pad / 128) * ceil_div(r, 128), h.n_d);
 }
 static int64_t head_slices_t(const dense_head& h, int r, int64_t n) {
-  return ptq_slices((h.n_d_pad / 128) * ceil_div(r, 128), ceil_div(n, PTQ_KB));
+  return head_slices_for((h.n_d_pad / 128) * ceil_div(r, 128), n);
 }
 
 int head_ensure_workspace(dnpeff_csr* A, int r) {
@@ -521,8 +530,22 @@ int head_ensure_workspace(dnpeff_csr* A, int r) {
   const int64_t wt = head_slices_t(h, r, A->n_rows) * h.n_d_pad * r;
   const int64_t need = gather + (wn > wt ? wn : wt);
   if (!head_uses_split(r) && !h.rm) {  // the fp32 kernel of A^T W wants the block row by row
-    DN_TRY(dmalloc(&h.rm, h.n_pad * h.n_d_pad));
-    DN_TRY(launch_transpose(h.n_d_pad, h.n_pad, h.cm, h.rm));
+    if (dmalloc(&h.rm, h.n_pad * h.n_d_pad)) {
+      // no room for the second copy: at ranks that the split-operand kernel handles the head's
+      // share of A^T W stays on it (said once), other ranks cannot go on
+      h.rm = nullptr;
+      DN_CHECK(r % 128 == 0, "dense head: no memory for the row-major block (%lld bytes)",
+               (long long)(4 * h.n_pad * h.n_d_pad));
+      clear_error();
+      static bool told = false;
+      if (!told) {
+        told = true;
+        fprintf(stderr, "dnpeff: no memory for the row-major copy of the dense head: its share of A^T W "
+                        "stays on the split-operand kernel\n");
+      }
+    } else {
+      DN_TRY(launch_transpose(h.n_d_pad, h.n_pad, h.cm, h.rm));
+    }
   }
   if (h.ws && h.ws_floats >= need) return 0;
   dfree(h.ws);
@@ -570,7 +593,7 @@ int launch_head_t_product(const dnpeff_csr* A, int r, const float* W_nr) {
   DN_CHECK(h.ws && r % 4 == 0 && ((uintptr_t)W_nr % 16) == 0, "dense head: workspace or alignment");
   float* part = h.ws + head_gather_floats(h, r);
   const int64_t slices = head_slices_t(h, r, A->n_rows);
-  if (head_uses_split(r)) {
+  if (head_uses_split(r) || (r % 128 == 0 && !h.rm)) {
     // D^T [n_d, n] (cm) times W transposed: contraction over the rows of the matrix
     float* Wt = h.ws;
     dim3 tg((unsigned)ceil_div(h.n_pad, 32), (unsigned)ceil_div(r, 32));

@@ -185,19 +185,32 @@ inline hid_t write_1d(hid_t grp, const char* name, hid_t type, const T* data, si
   return ds;
 }
 
-// NmfDecomposition<int32_t>::save (nmf_decomp_h5.h:38-89): data/W [n, r], data/H [r, m],
-// data/reduce_kept_indices [m] with attribute full_dense_size of shape (1,).
+// NmfDecomposition<IndT>::save (nmf_decomp_h5.h:38-89): data/W [n, r], data/H [r, m],
+// data/reduce_kept_indices [m] with attribute full_dense_size of shape (1,).  wide_indices:
+// both are written as int64, as the reference's IndT = int64_t instantiation does (the main
+// selects it when n_examples x n_fisher_values exceeds INT32_MAX, pef_fisher_h5.h:57-90).
 inline void write_dense_decomposition(const std::string& path, long n, long r, long m, const float* W,
-                                      const float* H, const int32_t* kept, int32_t full_dense_size) {
+                                      const float* H, const int32_t* kept, int64_t full_dense_size,
+                                      bool wide_indices = false) {
   hid_t file = check(H5Fcreate(path.c_str(), H5F_ACC_TRUNC, H5P_DEFAULT, H5P_DEFAULT), "create " + path);
   hid_t data = check(H5Gcreate(file, "data", H5P_DEFAULT, H5P_DEFAULT, H5P_DEFAULT), "group data");
   write_matrix(data, "W", n, r, W);
   write_matrix(data, "H", r, m, H);
-  hid_t ds = write_1d(data, "reduce_kept_indices", H5T_NATIVE_INT32, kept, (size_t)m, false);
+  hid_t ds;
   hsize_t one[1] = {1};
   hid_t sp = H5Screate_simple(1, one, one);
-  hid_t a = check(H5Acreate(ds, "full_dense_size", H5T_NATIVE_INT32, sp, H5P_DEFAULT, H5P_DEFAULT), "full_dense_size");
-  check_status(H5Awrite(a, H5T_NATIVE_INT32, &full_dense_size), "write full_dense_size");
+  hid_t a;
+  if (wide_indices) {
+    std::vector<int64_t> kept64(kept, kept + m);
+    ds = write_1d(data, "reduce_kept_indices", H5T_NATIVE_INT64, kept64.data(), (size_t)m, false);
+    a = check(H5Acreate(ds, "full_dense_size", H5T_NATIVE_INT64, sp, H5P_DEFAULT, H5P_DEFAULT), "full_dense_size");
+    check_status(H5Awrite(a, H5T_NATIVE_INT64, &full_dense_size), "write full_dense_size");
+  } else {
+    const int32_t fds = (int32_t)full_dense_size;
+    ds = write_1d(data, "reduce_kept_indices", H5T_NATIVE_INT32, kept, (size_t)m, false);
+    a = check(H5Acreate(ds, "full_dense_size", H5T_NATIVE_INT32, sp, H5P_DEFAULT, H5P_DEFAULT), "full_dense_size");
+    check_status(H5Awrite(a, H5T_NATIVE_INT32, &fds), "write full_dense_size");
+  }
   H5Aclose(a);
   H5Sclose(sp);
   H5Dclose(ds);

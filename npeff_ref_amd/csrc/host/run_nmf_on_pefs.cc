@@ -31,6 +31,7 @@ struct ProgramFlags {
   float eps = 1e-8f;
   long seed = 43190432042L;
   int log_every = 10;
+  int index_width = 0;  // 0: the reference's rule (64 when n_examples x n_fisher_values exceeds INT32_MAX)
 };
 
 static ProgramFlags parse_flags(int argc, char** argv) {
@@ -49,6 +50,7 @@ static ProgramFlags parse_flags(int argc, char** argv) {
   f.read("eps", &p.eps, false);
   f.read("seed", &p.seed, false);
   f.read("log_every", &p.log_every, false);
+  f.read("index_width", &p.index_width, false);
   return p;  // unknown flags are ignored, as in the reference
 }
 
@@ -57,8 +59,13 @@ int main(int argc, char** argv) {
 
   h5io::PefDims dims = h5io::pef_dims(flags.pef_path, flags.n_examples, flags.n_fisher_values);
   const long nnz_in = dims.n_rows * dims.n_values_per_row;
-  // Row offsets are always 64-bit and column ids 32-bit here; the line is kept for log parity.
-  if (nnz_in > (long)INT32_MAX)
+  // Row offsets are always 64-bit and column ids 32-bit inside the library; the reference's
+  // choice of index type (run_nmf_on_pefs.cu:236-244) still decides the log line and the type of
+  // reduce_kept_indices / full_dense_size in the output file (nmf_decomp_h5.h:58-75).
+  if (flags.index_width != 0 && flags.index_width != 32 && flags.index_width != 64)
+    fatal("Error: --index_width must be 32 or 64.");
+  const bool wide_indices = flags.index_width ? flags.index_width == 64 : nnz_in > (long)INT32_MAX;
+  if (wide_indices)
     std::cout << "Reading in PEFs using 64 bit indices.\n";
   else
     std::cout << "Using 32 bit indices.\n";
@@ -88,7 +95,8 @@ int main(int argc, char** argv) {
 
   std::cout << "Initializing NMF.\n";
   dnpeff_nmf* nmf = nullptr;
-  ck(dnpeff_nmf_create(A, flags.n_components, flags.eps, flags.seed, &nmf));
+  // the matrix is only asked for its column map afterwards: the context may take its arrays
+  ck(dnpeff_nmf_create_ex(A, flags.n_components, flags.eps, flags.seed, DNPEFF_NMF_CONSUME_MATRIX, &nmf));
   ck(dnpeff_nmf_init_factors(nmf));
   ck(dnpeff_sync());
 
@@ -120,8 +128,8 @@ int main(int argc, char** argv) {
   ck(dnpeff_csr_full_dense_size(A, &full));
 
   std::cout << "Saving decomposition to file.\n";
-  h5io::write_dense_decomposition(flags.output_path, n, r, m, W.data(), H.data(), kept.data(),
-                                  (int32_t)full);
+  h5io::write_dense_decomposition(flags.output_path, n, r, m, W.data(), H.data(), kept.data(), full,
+                                  wide_indices);
   dnpeff_nmf_destroy(nmf);
   dnpeff_csr_destroy(A);
   return 0;

@@ -1378,6 +1378,15 @@ DN_API int dnpeff_op_gather_rows(int64_t count, int r, const float* X, const int
   return 0;
 }
 
+// out[k] = cm[k * n_pad + row]: one row of the dense head's block
+__global__ void __launch_bounds__(256)
+    k_head_row(const float* __restrict__ cm, int64_t n_pad, int64_t row, int64_t n_d,
+               float* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x; k < n_d; k += stride)
+    out[k] = cm[k * n_pad + row];
+}
+
 // Entries of one row / one column of the matrix as the products hold it: the dense head's block
 // plus the sparse part (its regrouped or plain row-major copy, its transposed copy).
 DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* count, int32_t* cols,
@@ -1400,8 +1409,13 @@ DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* 
   if (A->head.n_d) {
     head_row.resize((size_t)A->head.n_d);
     head_cols.resize((size_t)A->head.n_d);
-    DN_HIP(hipMemcpy2D(head_row.data(), sizeof(float), A->head.cm + row, sizeof(float) * A->head.n_pad,
-                       sizeof(float), (size_t)A->head.n_d, hipMemcpyDeviceToHost));
+    dbuf<float> tmp;
+    DN_TRY(tmp.alloc(A->head.n_d));
+    hipLaunchKernelGGL(k_head_row, dim3(grid_for(A->head.n_d, 4096)), dim3(256), 0, stream(), A->head.cm,
+                       A->head.n_pad, row, A->head.n_d, tmp.p);
+    DN_LAUNCH_CHECK();
+    DN_HIP(hipStreamSynchronize(stream()));
+    DN_HIP(hipMemcpy(head_row.data(), tmp.p, sizeof(float) * A->head.n_d, hipMemcpyDeviceToHost));
     DN_HIP(hipMemcpy(head_cols.data(), A->head.cols, sizeof(int32_t) * A->head.n_d,
                      hipMemcpyDeviceToHost));
     for (float v : head_row) got += v != 0.0f;

@@ -115,6 +115,35 @@ def test_run_nmf_on_pefs_end_to_end(tmp_path):
 
 
 @pytest.mark.gpu
+def test_run_nmf_on_pefs_wide_index_schema(tmp_path):
+    """The reference instantiates its writer with IndT = int64 when n_examples x n_fisher_values
+    exceeds INT32_MAX (nmf_decomp_h5.h:58-75): reduce_kept_indices and full_dense_size are then
+    int64.  --index_width=64 forces that branch on a small file; the values are the same, and
+    the fit path reads such a file."""
+    n, m_full, k, r = 24, 9000, 300, 8
+    pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=5)
+    out32, out64 = str(tmp_path / "d32.h5"), str(tmp_path / "d64.h5")
+    common = [f"--per_example_fishers={pef}", f"--nmf_n_components={r}", "--nmf_max_iter=3"]
+    run("run_nmf_on_pefs", f"--output_path={out32}", *common, check=True)
+    p = run("run_nmf_on_pefs", f"--output_path={out64}", "--index_width=64", *common, check=True)
+    assert "Reading in PEFs using 64 bit indices." in p.stdout.splitlines()
+    k32, k64 = h5lite.read(out32, "data/reduce_kept_indices"), h5lite.read(out64, "data/reduce_kept_indices")
+    assert k32.dtype == np.int32 and k64.dtype == np.int64 and np.array_equal(k32, k64)
+    f32, s32 = h5lite.attr(out32, "data/reduce_kept_indices", "full_dense_size")
+    f64, s64 = h5lite.attr(out64, "data/reduce_kept_indices", "full_dense_size")
+    assert f32.dtype == np.int32 and f64.dtype == np.int64 and s32 == s64 == (1,)
+    assert int(f32[0]) == int(f64[0]) == m_full
+    assert np.array_equal(h5lite.read(out32, "data/H"), h5lite.read(out64, "data/H"))
+    # the sparsifier reads the wide file as it reads the narrow one
+    sp32, sp64 = str(tmp_path / "s32.h5"), str(tmp_path / "s64.h5")
+    run("sparsify_d_npeff", f"--decomposition_filepath={out32}", f"--output_filepath={sp32}", "--H_threshold=1e-3",
+        check=True)
+    run("sparsify_d_npeff", f"--decomposition_filepath={out64}", f"--output_filepath={sp64}", "--H_threshold=1e-3",
+        check=True)
+    assert np.array_equal(h5lite.read(sp32, "data/H/values"), h5lite.read(sp64, "data/H/values"))
+
+
+@pytest.mark.gpu
 def test_fit_coeffs_to_sparse_H_end_to_end(tmp_path):
     n, m_full, k, r, iters = 50, 20000, 400, 8, 50
     pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=21, sparse_H_output_path=str(tmp_path / "H.h5"), rank=r,
