@@ -315,6 +315,10 @@ def run_nmf(d, args, cfg):
     nmf.step(args.warmup)
     d.sync()
     loss_before = nmf.computeUncachedLoss()
+    # (the loss leaves A H^T behind for the next W update: one more untimed step, so that every
+    # timed step computes both products)
+    nmf.step(1)
+    d.sync()
     nmf.set_profiling(True)
     nmf.timings(reset=True)
     d.sync()

@@ -534,6 +534,7 @@ int head_ensure_workspace(dnpeff_csr* A, int r) {
       // no room for the second copy: at ranks that the split-operand kernel handles the head's
       // share of A^T W stays on it (said once), other ranks cannot go on
       h.rm = nullptr;
+      (void)hipGetLastError();  // (the failed allocation must not surface at the next launch check)
       DN_CHECK(r % 128 == 0, "dense head: no memory for the row-major block (%lld bytes)",
                (long long)(4 * h.n_pad * h.n_d_pad));
       clear_error();
