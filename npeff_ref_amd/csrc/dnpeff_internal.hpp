@@ -253,6 +253,8 @@ constexpr int SWEEP_XCDS = 8;
 inline int64_t panel_slots(const dnpeff_csr* S) {
   return S->n_plain + (S->n_swept > 0 ? SWEEP_XCDS : 0);
 }
+// Whether the workgroups of a launch go to the SWEEP_XCDS XCDs round-robin (probed once).
+bool xcd_round_robin();
 // Ranks the sweep kernel of A H^T handles.
 inline bool spmm_n_sweep_supported(int r) { return r == 32 || r == 64 || r == 128 || r == 256; }
 // Everything A H^T and A^T W at rank r need: transposed copy and work lists of the sparse part,

@@ -80,6 +80,45 @@ tuning_t& tuning() {
   return t;
 }
 
+// ids[b] = XCD that workgroup b of the probe runs on (hardware register XCC_ID, bits 3:0)
+__global__ void k_xcd_probe(int* ids) {
+  if (threadIdx.x == 0) ids[blockIdx.x] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15;
+}
+
+// The kernels that pin work to an XCD (swept pieces of A H^T, component slices of A^T W) count on
+// the dispatcher dealing the workgroups of a launch to SWEEP_XCDS XCDs round-robin by their
+// number: workgroups b, b + 8, b + 16, ... on one XCD, the eight classes on eight different ones
+// (which XCD a class gets does not matter).  Checked once per process with a probe launch; where
+// it does not hold (another partition mode, another part) those plans are not made: plain
+// panels, one slice.
+bool xcd_round_robin() {
+  static int state = -1;
+  if (state >= 0) return state == 1;
+  state = 0;
+  constexpr int N = 64 * SWEEP_XCDS;
+  int* ids = nullptr;
+  if (dmalloc(&ids, N)) return false;
+  int h[N];
+  hipLaunchKernelGGL(k_xcd_probe, dim3(N), dim3(64), 0, stream(), ids);
+  if (hipGetLastError() == hipSuccess &&
+      hipMemcpy(h, ids, sizeof(int) * N, hipMemcpyDeviceToHost) == hipSuccess) {
+    bool ok = true;
+    unsigned seen = 0;
+    for (int x = 0; x < SWEEP_XCDS; x++) {
+      for (int b = x; b < N; b += SWEEP_XCDS) ok = ok && h[b] == h[x];
+      ok = ok && !(seen & (1u << h[x]));
+      seen |= 1u << h[x];
+    }
+    state = ok ? 1 : 0;
+  }
+  dfree(ids);
+  clear_error();
+  if (state == 0 && tuning().verbose != 0.0)
+    fprintf(stderr, "dnpeff: workgroups are not dealt to %d XCDs round-robin: no swept pieces, no "
+                    "component slices\n", SWEEP_XCDS);
+  return state == 1;
+}
+
 struct KeepMaskF {
   const int* count;
   int min_count;
@@ -655,7 +694,7 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   const tuning_t& tn = tuning();
   int64_t P = 0;
   const double bytes = 4.0 * (double)S->n_cols * r;
-  const bool sweeps = spmm_n_sweep_supported(r) && tn.sweep_bytes > 0.0;
+  const bool sweeps = spmm_n_sweep_supported(r) && tn.sweep_bytes > 0.0 && xcd_round_robin();
   if (bytes >= 512e6 && S->n_rows >= 64) {
     // with swept pieces for the panels in between, half as many coarse panels do as well for the
     // gathers and halve the sum over the panels (configs[1]: 19.8 -> 19.4 ms for both)

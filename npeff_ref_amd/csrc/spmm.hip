@@ -1142,6 +1142,7 @@ static int spmm_t_slices(int64_t n, int r) {
   const int forced = (int)tuning().spmm_t_slices;
   if (forced == 1 || ((forced == 2 || forced == 4 || forced == 8) && ok(forced))) return forced;
   int v = 1;
+  if (!xcd_round_robin()) return v;  // slices pay through the XCDs' own L2s only
   while (v < 8 && ok(2 * v) && 4.0 * (double)n * r / v > 6.0e6) v *= 2;
   return v;
 }
