@@ -256,7 +256,15 @@ inline int64_t panel_slots(const dnpeff_csr* S) {
 // Whether the workgroups of a launch go to the SWEEP_XCDS XCDs round-robin (probed once).
 bool xcd_round_robin();
 // Ranks the sweep kernel of A H^T handles.
-inline bool spmm_n_sweep_supported(int r) { return r == 32 || r == 64 || r == 128 || r == 256; }
+// Components that one launch of the sweep kernel sums: the rank itself up to 256, else slices of
+// 256 or 128 components (0 = the rank has no sweep kernel).
+inline int sweep_width(int r) {
+  if (r == 32 || r == 64 || r == 128 || r == 256) return r;
+  if (r > 256 && r % 256 == 0) return 256;
+  if (r > 256 && r % 128 == 0) return 128;
+  return 0;
+}
+inline bool spmm_n_sweep_supported(int r) { return sweep_width(r) != 0; }
 // Everything A H^T and A^T W at rank r need: transposed copy and work lists of the sparse part,
 // workspaces of the sparse part and of the dense head.
 int csr_ensure_products(dnpeff_csr* A, int r);

@@ -714,7 +714,7 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   if (P > 0 && sweeps) {
     double sweep_bytes = tn.sweep_bytes;
     if (sweep_bytes > 1e9) sweep_bytes = 1e9;  // (the kernel addresses a piece with 32 bits)
-    plan.sweep_cols = (int)(sweep_bytes / (4.0 * r));
+    plan.sweep_cols = (int)(sweep_bytes / (4.0 * sweep_width(r)));  // (a piece of one slice)
     // a piece must also bring work enough for a sweep step (a wait for the other workgroups of
     // the XCD and two barriers): 20,000 entries over all rows
     plan.sweep_min = 4.0;

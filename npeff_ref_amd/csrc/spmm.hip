@@ -322,9 +322,12 @@ __global__ void __launch_bounds__(1024)
     k_spmm_n_sweep(const int64_t* __restrict__ seg, const int32_t* __restrict__ pcol,
                    const float* __restrict__ pval, int64_t row0, int64_t row1, int P,
                    const int32_t* __restrict__ swept, int n_swept,
-                   const int32_t* __restrict__ bounds_of, int slots, int slot0, int r,
+                   const int32_t* __restrict__ bounds_of, int slots, int slot0, int r, int stride,
                    const float* __restrict__ H, float* __restrict__ part,
                    int* __restrict__ progress, int lag, int spin_max, int rows_wg) {
+  // r: components that this launch sums (4 LPR); stride: floats between two rows of H and of
+  // the partial sums (the rank; r < stride for a launch on a slice of the components, whose H and
+  // part pointers then start at the slice's first component)
   extern __shared__ __align__(16) float sums[];  // [rows_wg][r], row l = i * waves + wave
   constexpr int G = 64 / LPR;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -359,7 +362,7 @@ __global__ void __launch_bounds__(1024)
     const int lo = (int)(uint32_t)(v & 0xffffffffLL), hi = (int)(v >> 32);
     return ((int64_t)bcast_i(hi, src) << 32) | (uint32_t)bcast_i(lo, src);
   };
-  const unsigned r4 = 4u * (unsigned)r, sub16 = 16u * (unsigned)sub;
+  const unsigned r4 = 4u * (unsigned)stride, sub16 = 16u * (unsigned)sub;
 
   if (n_pi > 0) {  // (n_pi is the same for all waves of the workgroup)
     int64_t cm_s0, st_s0;
@@ -376,7 +379,7 @@ __global__ void __launch_bounds__(1024)
     int pi = 0, i = 0;
     // rows of H of the current piece: Hp + 4 r (column - c0), a 32-bit offset
     int c0 = bounds_of[swept[x]];
-    const char* Hp = reinterpret_cast<const char*>(H + (int64_t)c0 * r);
+    const char* Hp = reinterpret_cast<const char*>(H + (int64_t)c0 * stride);
     int ra_i, rb_i;
     float ra_v, rb_v;
     ra_i = (pcol + bcast_i64(cm_s0, 0))[lane];
@@ -574,7 +577,7 @@ __global__ void __launch_bounds__(1024)
         pi++;
         load_off(pi + 2, st_s0, st_len);
         c0 = bounds_of[swept[x + SWEEP_XCDS * (pi < n_pi ? pi : 0)]];
-        Hp = reinterpret_cast<const char*>(H + (int64_t)c0 * r);
+        Hp = reinterpret_cast<const char*>(H + (int64_t)c0 * stride);
         __syncthreads();
         if (threadIdx.x == 0)
           __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -591,7 +594,7 @@ __global__ void __launch_bounds__(1024)
     const int64_t row = row_of(i);
     if (row < row1) {
       const float* src = sums + (size_t)(i * waves + wave) * r;
-      float* dst = part + (row * slots + slot0 + x) * r;
+      float* dst = part + (row * slots + slot0 + x) * stride;
       for (int c = lane; c < r; c += 64) dst[c] = src[c];
     }
   }
@@ -1011,9 +1014,11 @@ static sweep_shape sweep_shape_for(int64_t n_rows, int r, int max_waves) {
 constexpr int SWEEP_REGISTER_BUDGET = 448;
 
 using sweep_kernel_t = void (*)(const int64_t*, const int32_t*, const float*, int64_t, int64_t, int,
-                                const int32_t*, int, const int32_t*, int, int, int, const float*,
+                                const int32_t*, int, const int32_t*, int, int, int, int, const float*,
                                 float*, int*, int, int, int);
 
+// Ranks above 256 are swept in slices of 256 (or 128) components: one set of launches per slice,
+// each with its slice of every row of H pinned in the L2s and its own running sums.
 static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bool aligned,
                                int slots) {
   DN_CHECK(spmm_n_sweep_supported(r), "swept panels at rank %d", r);
@@ -1023,7 +1028,8 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
       k_spmm_n_sweep<16, true>,  k_spmm_n_sweep<32, false>, k_spmm_n_sweep<32, true>,
       k_spmm_n_sweep<64, false>, k_spmm_n_sweep<64, true>};
   static int kernel_regs[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // 0: attributes not yet set
-  const int variant = (r == 32 ? 0 : r == 64 ? 2 : r == 128 ? 4 : 6) + (aligned ? 1 : 0);
+  const int w = sweep_width(r);
+  const int variant = (w == 32 ? 0 : w == 64 ? 2 : w == 128 ? 4 : 6) + (aligned ? 1 : 0);
   const sweep_kernel_t kernel = kernels[variant];
   if (kernel_regs[variant] == 0) {
     hipFuncAttributes attr;
@@ -1038,32 +1044,33 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
   if (max_waves > 14) max_waves = 14;
   max_waves &= ~1;
   DN_CHECK(max_waves >= 2, "the sweep kernel needs %d registers", kernel_regs[variant]);
-  const sweep_shape sh = sweep_shape_for(A->n_rows, r, max_waves);
+  const sweep_shape sh = sweep_shape_for(A->n_rows, w, max_waves);
   DN_CHECK(sh.waves > 0, "no sweep shape for rank %d", r);
   static bool told = false;
   if (!told && tuning().verbose != 0.0) {
     told = true;
     fprintf(stderr,
             "dnpeff: sweep kernel with %d registers: %lld workgroups of %d waves, %d rows each, "
-            "%lld pass(es) of %lld rows\n",
+            "%lld pass(es) of %lld rows, %d slice(s) of %d components\n",
             kernel_regs[variant], (long long)sh.wgs, sh.waves, sh.rows_wg, (long long)sh.n_pass,
-            (long long)sh.rows_per_pass);
+            (long long)sh.rows_per_pass, r / w, w);
   }
   const int32_t* swept = A->panel_ids + A->n_plain;
   int lag = (int)tuning().sweep_lag, spin_max = (int)tuning().sweep_spin;
   if (lag < 0) lag = 0;
-  const size_t lds = sizeof(float) * (size_t)sh.rows_wg * r;
-  for (int64_t pass = 0; pass < sh.n_pass; pass++) {
-    const int64_t row0 = pass * sh.rows_per_pass;
-    const int64_t row1 = row0 + sh.rows_per_pass < A->n_rows ? row0 + sh.rows_per_pass : A->n_rows;
-    hipLaunchKernelGGL(k_sweep_clear, dim3(1), dim3(SWEEP_XCDS * SWEEP_SYNC_STRIDE), 0, stream(),
-                       A->sweep_progress);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)sh.wgs), dim3(64 * sh.waves), lds, stream(), A->seg,
-                       A->pcol, A->pval, row0, row1, A->n_panels, swept, A->n_swept,
-                       A->panel_bounds, slots, A->n_plain, r, H_mr, A->partials, A->sweep_progress,
-                       lag, spin_max, sh.rows_wg);
-    DN_LAUNCH_CHECK();
-  }
+  const size_t lds = sizeof(float) * (size_t)sh.rows_wg * w;
+  for (int slice = 0; slice < r / w; slice++)
+    for (int64_t pass = 0; pass < sh.n_pass; pass++) {
+      const int64_t row0 = pass * sh.rows_per_pass;
+      const int64_t row1 = row0 + sh.rows_per_pass < A->n_rows ? row0 + sh.rows_per_pass : A->n_rows;
+      hipLaunchKernelGGL(k_sweep_clear, dim3(1), dim3(SWEEP_XCDS * SWEEP_SYNC_STRIDE), 0, stream(),
+                         A->sweep_progress);
+      hipLaunchKernelGGL(kernel, dim3((unsigned)sh.wgs), dim3(64 * sh.waves), lds, stream(), A->seg,
+                         A->pcol, A->pval, row0, row1, A->n_panels, swept, A->n_swept,
+                         A->panel_bounds, slots, A->n_plain, w, r, H_mr + slice * w,
+                         A->partials + slice * w, A->sweep_progress, lag, spin_max, sh.rows_wg);
+      DN_LAUNCH_CHECK();
+    }
   return 0;
 }
 

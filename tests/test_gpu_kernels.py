@@ -358,6 +358,9 @@ def test_spmm_n_column_panels(panels, r, n, m, maxk, tune):
     (64, 200, 4000, 3000, 2, 300 * 256, 8),      # long segments at 4 lane groups (several batches of 64)
     (32, 150, 3000, 2500, 2, 400 * 128, 4),      # long segments at 8 lane groups (shuffles, no row broadcasts)
     (256, 120, 3000, 2800, 2, 500 * 1024, 6),    # long segments at one lane group (4 rows of 16 lanes)
+    (512, 90, 2000, 700, 2, 400 * 1024, 8),      # rank above 256: two slices of 256 components
+    (384, 70, 1500, 500, 3, 300 * 512, 4),       # three slices of 128
+    (1024, 40, 900, 400, 2, 200 * 1024, 2),      # four slices of 256
 ])
 def test_spmm_n_swept_panels(r, n, m, maxk, panels, sweep_bytes, waves, tune):
     """Coarse panels cut into L2-sized pieces that one XCD sweeps for all rows, running sums in
