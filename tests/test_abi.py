@@ -105,3 +105,41 @@ def test_generator_rejects_impossible_requests():
         d.synth_pef_host(2, 10, k_fixed=8)  # k > n_cols / 2
     with pytest.raises(d.DnpeffError):
         d.synth_pef_host(2, 1000, k_fixed=8, zipf_s=1.0)
+
+
+def test_tuning_switches_round_trip_and_reject_unknown_names():
+    assert d.tuning_get("sweep_spin") == 400.0
+    d.tuning_set("sweep_spin", 3)
+    assert d.tuning_get("sweep_spin") == 3.0
+    d.tuning_reset()
+    assert d.tuning_get("sweep_spin") == 400.0
+    with pytest.raises(d.DnpeffError, match="no tuning switch"):
+        d.tuning_set("no_such_switch", 1)
+    with pytest.raises(d.DnpeffError, match="no tuning switch"):
+        d.tuning_get("no_such_switch")
+
+
+def test_host_generator_row_range_matches_the_whole_matrix():
+    rowptr, colind, vals, norms = d.synth_pef_host(30, 80000, k_fixed=200, zipf_s=1.3, seed=9)
+    rp, ci, va, nr = d.synth_pef_host_rows(11, 4, 80000, k_fixed=200, zipf_s=1.3, seed=9)
+    assert rp.tolist() == [0, 200, 400, 600, 800]
+    assert np.array_equal(ci, colind[11 * 200:15 * 200]) and np.array_equal(va, vals[11 * 200:15 * 200])
+    assert np.array_equal(nr, norms[11:15])
+
+
+def test_bench_work_model_and_sample_sizes():
+    """bench.py's algorithmic bytes follow the formulas of the measurement plan, and the CPU
+    sample is the whole matrix for configs[1] and a few hundred rows for configs[3]."""
+    import bench
+
+    n, m, z, r = 20_000, 211_311_151, 5_242_880_000, 256
+    assert bench.algorithmic("spmm_n", n, m, z, r)[0] == 8 * z + 8 * (n + 1) + 4 * r * m + 4 * n * r
+    assert bench.algorithmic("spmm_t", n, m, z, r)[0] == 8 * z + 8 * (m + 1) + 4 * n * r + 4 * r * m
+    assert bench.algorithmic("spmm_n", 10, 100, 1000, 4)[0] == 8 * 1000 + 4 * 11 + 4 * 4 * 100 + 4 * 10 * 4
+    b, f, split = bench.algorithmic("xg_mu_H", n, m, z, r, split_bf16=True)
+    assert b == 12 * m * r + 4 * r * r and f == 2 * m * r * r and split
+    assert bench.cpu_sample_rows(bench.CONFIGS["c1"]) == 10_000
+    assert 256 <= bench.cpu_sample_rows(bench.CONFIGS["c3"]) <= 1024
+    assert bench.traffic_from_profile("c3", "spmm_n")[0] == pytest.approx(9.40e11)
+    assert bench.traffic_from_profile("c3", "no_such_class") == (None, None)
+    assert bench.traffic_from_profile("c0", "spmm_n") == (None, None)

@@ -25,12 +25,12 @@ pytestmark = pytest.mark.gpu
 TOL = 2e-5
 
 
-def _full_size_checks(n, m_full, k, zipf_s, r, seed, n_rows_sampled, tiled_expected):
-    A, norms = d.Csr.synth(n, m_full, k_fixed=k, zipf_s=zipf_s, seed=seed)
+def _full_size_checks(n, m_full, k, zipf_s, r, seed, n_rows_sampled, tiled_expected, k_min=0, k_max=0):
+    A, norms = d.Csr.synth(n, m_full, k_fixed=k, k_min=k_min, k_max=k_max, zipf_s=zipf_s, seed=seed)
     A.normalize_rows(norms)
     A.compact_columns(1)
     m, z = A.n_cols, A.nnz
-    assert z == n * k and A.full_dense_size == m_full
+    assert (z == n * k if k else n * k_min <= z <= n * k_max) and A.full_dense_size == m_full
     kept = A.kept_indices()
     assert np.all(np.diff(kept.astype(np.int64)) > 0)  # newToOgIndex ascends
     nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=0, eps=1e-12, seed=seed), consume_matrix=True)
@@ -77,20 +77,22 @@ def _full_size_checks(n, m_full, k, zipf_s, r, seed, n_rows_sampled, tiled_expec
     rows = np.unique(np.concatenate([[0, n // 3, n - 1], rng.integers(0, n, n_rows_sampled)]))[:n_rows_sampled]
     lookups = []
     for i in rows:
-        rp, ci, va, nr = d.synth_pef_host_rows(int(i), 1, m_full, k_fixed=k, zipf_s=zipf_s, seed=seed)
+        rp, ci, va, nr = d.synth_pef_host_rows(int(i), 1, m_full, k_fixed=k, k_min=k_min, k_max=k_max,
+                                               zipf_s=zipf_s, seed=seed)
+        k_row = len(ci)
         assert nr[0] == norms[i]  # host twin and device generator agree on the row
         want_cols = np.searchsorted(kept, ci).astype(np.int32)
         assert np.array_equal(kept[want_cols], ci)
         want_vals = (va / np.float32(nr[0] + np.float32(1e-9))).astype(np.float32)
         got_cols, got_vals = A.get_row(int(i))
-        assert len(got_cols) == k
+        assert len(got_cols) == k_row
         o_w, o_g = np.argsort(want_cols, kind="stable"), np.argsort(got_cols, kind="stable")
         assert np.array_equal(want_cols[o_w], got_cols[o_g])
         assert np.array_equal(want_vals[o_w], got_vals[o_g])  # bit-exact loader at this size
         Hrows = d.gather_rows(h_dev, r, want_cols).astype(np.float64)
         N64 = want_vals.astype(np.float64) @ Hrows
         assert np.max(np.abs(N[i] - N64)) <= TOL * np.max(np.abs(N64))
-        pick = rng.integers(0, k, 6)
+        pick = rng.integers(0, k_row, 6)
         lookups += [(int(i), int(want_cols[p]), want_vals[p]) for p in pick]
 
     # the transposed copy lists these entries too
@@ -131,3 +133,75 @@ def test_configs3_at_full_size():
         pytest.skip("configs[3] needs the 288 GB of an MI355X")
     _full_size_checks(20_000, 350_000_000, 262_144, 1.3, 256, 43190432042, n_rows_sampled=8,
                       tiled_expected=True)
+
+
+@pytest.mark.timeout(600)
+def test_configs4_ragged_rows_at_full_size():
+    """configs[4]: 40,000 rows of 1,024 ... 524,288 entries (3.34e9 in all) x 110M, r = 512."""
+    free, total = d.device_memory()
+    if total < 280e9:
+        pytest.skip("configs[4] needs the 288 GB of an MI355X")
+    _full_size_checks(40_000, 110_000_000, 0, 1.1, 512, 43190432042, n_rows_sampled=6, tiled_expected=True,
+                      k_min=1_024, k_max=524_288)
+
+
+def test_configs2_fit_path_at_full_size():
+    """configs[2]: 50,000 new examples x 65,536 entries (3.28e9, past 2^31) against a fixed sparse
+    H of rank 256 over 110M features at 1 % density.  First stage: sampled rows of A H^T and the
+    whole of H H^T against fp64 sums on the host; second stage: the W update works row by row, so
+    the sampled rows are followed on the host in fp64 from the same seeded start, and the logged
+    loss is the reference's (stale W H H^T) formula on the device's own products."""
+    from oracle import oracle as orc
+
+    n, m, k, r, seed = 50_000, 110_000_000, 65_536, 256, 43190432042
+    rng = np.random.default_rng(3)
+    rp, cols = [0], []
+    for _ in range(r):  # every entry present with probability 0.01: geometric gaps
+        idx = np.cumsum(rng.geometric(0.01, size=int(m * 0.0105) + 64)) - 1
+        idx = idx[idx < m].astype(np.int32)
+        cols.append(idx)
+        rp.append(rp[-1] + len(idx))
+    hci = np.concatenate(cols)
+    hva = np.exp(rng.normal(-8.0, 2.0, size=len(hci))).astype(np.float32)
+    hrp = np.array(rp, dtype=np.int64)
+    H = d.Csr.from_host(hrp, hci, hva, m)
+    A, norms = d.Csr.synth(n, m, k_fixed=k, zipf_s=1.1, seed=seed)
+    A.normalize_rows(norms)
+    assert A.nnz == n * k > 2**31
+    L = d.Learner(A, H, d.LearnerParams(max_iters=0, eps=1e-7, seed=seed))
+    AH, HH, sq = L.products()
+    assert abs(sq - n) < 1e-3 * n  # rows are L2-normalised
+    # H H^T in fp64 from H's rows (sorted columns: intersections by searchsorted)
+    for a, b in [(0, 0), (3, 200), (255, 17), (100, 100)]:
+        ca, va_ = hci[hrp[a]:hrp[a + 1]], hva[hrp[a]:hrp[a + 1]].astype(np.float64)
+        cb, vb_ = hci[hrp[b]:hrp[b + 1]], hva[hrp[b]:hrp[b + 1]].astype(np.float64)
+        pos = np.searchsorted(cb, ca)
+        hit = (pos < len(cb)) & (cb[np.minimum(pos, len(cb) - 1)] == ca)
+        want = float(np.sum(va_[hit] * vb_[pos[hit]]))
+        assert abs(HH[a, b] - want) <= 2e-5 * max(abs(want), 1e-30)
+        assert abs(HH[a, b] - HH[b, a]) <= 1e-6 * abs(want)  # (two sums of the same terms in another order)
+    # sampled rows of A H^T: the row made again on the host, H's columns looked up in its CSC
+    colptr, comp, tv = orc.transpose(hrp, hci, hva, m)
+    rows = [0, 1, n // 2, n - 1] + list(rng.integers(0, n, 12))
+    for i in rows:
+        rpi, ci, va, nr = d.synth_pef_host_rows(int(i), 1, m, k_fixed=k, zipf_s=1.1, seed=seed)
+        v = (va / np.float32(nr[0] + np.float32(1e-9))).astype(np.float64)
+        want = np.zeros(r)
+        lens = colptr[ci.astype(np.int64) + 1] - colptr[ci]
+        for e in np.nonzero(lens)[0]:
+            p0, p1 = colptr[ci[e]], colptr[ci[e] + 1]
+            np.add.at(want, comp[p0:p1], v[e] * tv[p0:p1].astype(np.float64))
+        assert np.max(np.abs(AH[i] - want)) <= 2e-5 * np.max(np.abs(want))
+    # second stage on the sampled rows
+    L.initialize()
+    L.step(25)
+    W = L.GetOnHost_W()
+    ref_loss, true_loss = L.losses()
+    sel = np.array(sorted(set(int(x) for x in rows)))
+    W0 = np.array([[d.uniform_at(seed, 0, i, c, r) for c in range(r)] for i in sel], dtype=np.float32)
+    W64, _, _ = orc.fit_f64(AH[sel], HH, 1.0, W0, np.float32(1e-7), 25, log_every=0)
+    assert np.linalg.norm(W[sel] - W64) / np.linalg.norm(W64) < 1e-4
+    assert np.isfinite(W).all() and W.min() >= 0 and np.isfinite([ref_loss, true_loss]).all()
+    L.close()
+    A.close()
+    H.close()

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import npeff_ref_amd as d
-from conftest import random_csr
+from conftest import csr_to_dense, random_csr
 from oracle import oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -445,3 +445,60 @@ def test_topk_rows_bit_exact(n, count, k, cap, tune):
     wv, wi, wn = orc.topk_rows(x, k)
     assert np.array_equal(v, wv) and np.array_equal(i, wi)
     assert np.all(np.abs(nrm - wn) <= 1e-6 * wn)
+
+
+def test_row_and_column_inspection_and_gathered_rows():
+    """dnpeff_csr_get_row / get_column return the matrix as the products hold it (dense head +
+    sparse part), before and after a consuming create; dnpeff_op_gather_rows picks rows of a factor;
+    the host generator's row range equals the rows of the whole matrix."""
+    rng = np.random.default_rng(17)
+    n, m, r = 1100, 9000, 64
+    rp, ci, va, hot = _hot_column_matrix(rng, n, m, 120, 60)
+    A = d.Csr.from_host(rp, ci, va, m)
+    assert A.split_dense_head(0.5) == 120
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=0), consume_matrix=True)
+    dense = csr_to_dense(rp, ci, va, m, dtype=np.float32)
+    for i in (0, 1, n // 2, n - 1):
+        cols, vals = A.get_row(i)
+        o = np.argsort(cols, kind="stable")
+        want = np.nonzero(dense[i])[0]
+        assert np.array_equal(cols[o], want) and np.array_equal(vals[o], dense[i, want])
+    for j in list(hot[:3]) + [0, 5, m - 1] + list(rng.integers(0, m, 20)):
+        rows, vals = A.get_column(int(j))
+        want = np.nonzero(dense[:, j])[0]
+        assert np.array_equal(rows, want) and np.array_equal(vals, dense[want, j])
+    nmf.initialize()
+    w_dev, h_dev = nmf.device_factors()
+    H = nmf.loadHToHostSync()
+    pick = np.array([5, 0, m - 1, 5, 77], dtype=np.int32)
+    assert np.array_equal(d.gather_rows(h_dev, r, pick), H[:, pick].T)
+    nmf.close()
+    A.close()
+    rowptr, colind, vals, norms = d.synth_pef_host(40, 50000, k_min=16, k_max=600, seed=4)
+    rp2, ci2, va2, nr2 = d.synth_pef_host_rows(7, 9, 50000, k_min=16, k_max=600, seed=4)
+    assert np.array_equal(rp2, rowptr[7:17] - rowptr[7])
+    assert np.array_equal(ci2, colind[rowptr[7]:rowptr[16]]) and np.array_equal(va2, vals[rowptr[7]:rowptr[16]])
+    assert np.array_equal(nr2, norms[7:16])
+
+
+@pytest.mark.parametrize("r", [64, 100, 512])
+def test_spmm_n_decompositions_agree(r, tune):
+    """One wave per row, 2048-entry row chunks and the planned decomposition (forced panels and
+    swept pieces) of A H^T on ragged rows: the same sums up to fp32 order, each against fp64."""
+    tune("panels", 8)
+    tune("sweep_bytes", 300 * 4 * min(r, 256))
+    tune("sweep_min", 0)
+    rowptr, colind, vals, norms = d.synth_pef_host(300, 40000, k_min=8, k_max=6000, seed=r)
+    A = d.Csr.from_host(rowptr, colind, vals, 40000)
+    rng = np.random.default_rng(r)
+    H = rng.random((40000, r)).astype(np.float32)
+    dH, dN = d.DeviceArray.from_numpy(H), d.DeviceArray((300, r))
+    N64 = orc.spmm_n_f64(rowptr, colind, vals, H)
+    for variant in (1, 2, 0):
+        d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, dH.ptr, dN.ptr, variant))
+        d.sync()
+        N = dN.numpy()
+        assert (np.abs(N - N64).max(axis=1) / np.maximum(np.abs(N64).max(axis=1), 1e-30)).max() < TOL
+    with pytest.raises(d.DnpeffError, match="variant"):
+        d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, dH.ptr, dN.ptr, 7))
+    A.close()
