@@ -11,13 +11,25 @@ constexpr int ABT_KB = 32;
 constexpr int ABT_LD = 80;                // bytes per row of a plane: 32 bf16 + 16 of padding
 constexpr int ABT_PLANE = 128 * ABT_LD;   // one part of one operand tile
 constexpr int ABT_LDS = 6 * ABT_PLANE;    // A: h, m, l; B: h, m, l
+#ifndef ABT_STAGES_XG
+#define ABT_STAGES_XG 2
+#endif
+#ifndef ABT_STAGES_ABT
+#define ABT_STAGES_ABT 2
+#endif
+#ifndef ABT_STAGES_GRAM
+#define ABT_STAGES_GRAM 2
+#endif
 
 // One operand tile (128 rows x 32 contraction elements) on its way from global memory to the
-// three bf16 planes in LDS.  KN = false: the source has the contraction index fast
-// (src[row * ld + k]): a thread takes 16 bytes of 4 rows, 8 threads per row.  KN = true: the
-// source has it slow (src[k * ld + row], e.g. a tile of X for X^T X): a thread takes 16
-// contraction elements of one row with 4-byte loads that are coalesced across the lanes, and
-// four consecutive ones make one 8-byte LDS store either way.
+// three bf16 planes in LDS, 16-byte loads either way.  KN = false: the source has the
+// contraction index fast (src[row * ld + k]): a thread takes 4 contraction elements of 4 rows,
+// 8 threads per row.  KN = true: the source has it slow (src[k * ld + row], e.g. a tile of X for
+// X^T X): a thread takes a 4 x 4 block, 4 rows of each of 4 consecutive contraction elements, and
+// turns it in registers; 8 consecutive threads hold the 32 contraction elements of 4 rows, so
+// that their LDS stores fall into different banks.  (With 4-byte loads, 16 per thread, the
+// address unit and not the matrix cores set the pace of X^T X.)  Either way four consecutive
+// contraction elements of a row make one 8-byte LDS store per part.
 template <bool KN>
 struct AbtOperand {
   f32x4 r[4];
@@ -28,26 +40,25 @@ struct AbtOperand {
       for (int q = 0; q < 4; q++)
         r[q] = *reinterpret_cast<const f32x4*>(src + (int64_t)(fr + 32 * q) * ld + k0 + fk);
     } else {
-      const int row = threadIdx.x & 127, kq = threadIdx.x >> 7;
-      const float* p = src + (k0 + 16 * kq) * ld + row;
+      const int row4 = 4 * (threadIdx.x >> 3), kb = 4 * (threadIdx.x & 7);
+      const float* p = src + (k0 + kb) * ld + row4;
 #pragma unroll
-      for (int q = 0; q < 4; q++)
-#pragma unroll
-        for (int u = 0; u < 4; u++) r[q][u] = p[(int64_t)(4 * q + u) * ld];
+      for (int q = 0; q < 4; q++) r[q] = *reinterpret_cast<const f32x4*>(p + q * ld);
     }
   }
   __device__ __forceinline__ void commit(unsigned char* planes) const {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       bf16x4 h, m, l;
-      split3(r[q], h, m, l);
       unsigned char* dst;
       if constexpr (!KN) {
         const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
+        split3(r[q], h, m, l);
         dst = planes + (fr + 32 * q) * ABT_LD + 2 * fk;
       } else {
-        const int row = threadIdx.x & 127, kq = threadIdx.x >> 7;
-        dst = planes + row * ABT_LD + 2 * (16 * kq + 4 * q);
+        const int row4 = 4 * (threadIdx.x >> 3), kb = 4 * (threadIdx.x & 7);
+        split3(f32x4{r[0][q], r[1][q], r[2][q], r[3][q]}, h, m, l);
+        dst = planes + (row4 + q) * ABT_LD + 2 * kb;
       }
       *reinterpret_cast<bf16x4*>(dst) = h;
       *reinterpret_cast<bf16x4*>(dst + ABT_PLANE) = m;
@@ -57,33 +68,36 @@ struct AbtOperand {
 };
 
 // acc += A B^T over the contraction tiles first, first + stride, ... (n_tiles of them).  Wave
-// (wm, wn) of the four owns the 64 x 64 quarter of the tile: blocks (i, j) of 32 x 32.  The next
-// contraction tile travels in registers while the 48 MFMAs of the current one run; every fp32
-// element is split once, on its way into LDS.  The sources must be readable for whole tiles
-// (zero padding, or rows clamped by the caller's pointer arithmetic).
-template <bool A_KN, bool B_KN>
+// (wm, wn) of the four owns the 64 x 64 quarter of the tile: blocks (i, j) of 32 x 32.  STAGES
+// contraction tiles travel in registers while the 48 MFMAs of the current one run (one tile of
+// MFMAs lasts 0.65 us, a trip to HBM three or four times that), and every fp32 element is split
+// once, on its way into LDS.  The loads are unconditional, so that the waits for them are counted
+// exactly: past the last tile they fetch the last one again.  The sources must be readable for
+// whole tiles (zero padding, or rows clamped by the caller's pointer arithmetic); with A_KN /
+// B_KN the source and its leading dimension must be 16-byte aligned.
+template <bool A_KN, bool B_KN, int STAGES = 1>
 __device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, int64_t lda,
                                              const float* __restrict__ b_src, int64_t ldb,
                                              int64_t first, int64_t stride, int64_t n_tiles,
                                              unsigned char* ab, abt_acc16 (&acc)[2][2]) {
+  static_assert(STAGES == 1 || STAGES == 2, "one or two tiles in registers");
+  if (n_tiles <= 0) return;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l32 = lane & 31, half = lane >> 5, wm = wave >> 1, wn = wave & 1;
-  AbtOperand<A_KN> oa;
-  AbtOperand<B_KN> ob;
-  if (n_tiles > 0) {
-    oa.fetch(a_src, lda, first * ABT_KB);
-    ob.fetch(b_src, ldb, first * ABT_KB);
-    oa.commit(ab);
-    ob.commit(ab + 3 * ABT_PLANE);
-  }
-  __syncthreads();
+  AbtOperand<A_KN> oa[STAGES];
+  AbtOperand<B_KN> ob[STAGES];
+  auto fetch = [&](int s, int64_t t) {
+    const int64_t k0 = (first + (t < n_tiles ? t : n_tiles - 1) * stride) * ABT_KB;
+    oa[s].fetch(a_src, lda, k0);
+    ob[s].fetch(b_src, ldb, k0);
+  };
+  auto commit = [&](int s) {
+    oa[s].commit(ab);
+    ob[s].commit(ab + 3 * ABT_PLANE);
+  };
   const unsigned char* a_row = ab + (64 * wm + l32) * ABT_LD + 16 * half;
   const unsigned char* b_row = ab + 3 * ABT_PLANE + (64 * wn + l32) * ABT_LD + 16 * half;
-  for (int64_t t = 0; t < n_tiles; t++) {
-    if (t + 1 < n_tiles) {
-      oa.fetch(a_src, lda, (first + (t + 1) * stride) * ABT_KB);
-      ob.fetch(b_src, ldb, (first + (t + 1) * stride) * ABT_KB);
-    }
+  auto mfma_tile = [&]() {
 #pragma unroll
     for (int st = 0; st < 2; st++) {
       bf16x8 ah[2], am[2], al[2], bh[2], bm[2], bl[2];
@@ -124,12 +138,25 @@ __device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, in
 #pragma unroll
         for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bm[j], acc[i][j]);
     }
-    __syncthreads();  // every wave is done with the planes
-    if (t + 1 < n_tiles) {
-      oa.commit(ab);
-      ob.commit(ab + 3 * ABT_PLANE);
+  };
+  // At the top of tile t: the planes hold tile t, and register stage (t + 1 + s) % STAGES holds
+  // tile t + 1 + s for s = 0 ... STAGES - 1 (requested, maybe not arrived).
+  fetch(0, 0);
+  commit(0);
+#pragma unroll
+  for (int s = 0; s < STAGES; s++) fetch((1 + s) % STAGES, 1 + s);
+  __syncthreads();
+  for (int64_t t = 0; t < n_tiles; t += STAGES) {
+#pragma unroll
+    for (int u = 0; u < STAGES; u++) {
+      if (t + u < n_tiles) {
+        mfma_tile();
+        __syncthreads();  // every wave is done with the planes
+        commit((u + 1) % STAGES);
+        fetch((u + 1) % STAGES, t + u + 1 + STAGES);
+        __syncthreads();
+      }
     }
-    __syncthreads();
   }
 }
 

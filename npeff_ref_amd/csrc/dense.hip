@@ -1022,7 +1022,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-  abt_mainloop<false, false>(X + row0 * r, r, Gt + (int64_t)n0 * r, r, 0, 1, r / ABT_KB, ab, acc);
+  abt_mainloop<false, false, ABT_STAGES_XG>(X + row0 * r, r, Gt + (int64_t)n0 * r, r, 0, 1, r / ABT_KB, ab, acc);
 
   auto finish = [&](int blk, const float (&n_)[16], const float (&x_)[16]) {
     const int i = blk >> 1, j = blk & 1;

@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-  abt_mainloop<A_KN, false>(A_KN ? A + m0 : A + m0 * lda, lda, B + (int64_t)n0 * ldb, ldb, z, S, n_my, ab,
+  abt_mainloop<A_KN, false, ABT_STAGES_ABT>(A_KN ? A + m0 : A + m0 * lda, lda, B + (int64_t)n0 * ldb, ldb, z, S, n_my, ab,
                             acc);
 
   // D layout of a 32x32 block: reg v of lane l holds row 8 (v/4) + 4 (l/32) + v%4, column l%32;
@@ -381,7 +381,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-  abt_mainloop<true, true>(X + 128 * ti, r, X + 128 * tj, r, z, S, n_my, ab, acc);
+  abt_mainloop<true, true, ABT_STAGES_GRAM>(X + 128 * ti, r, X + 128 * tj, r, z, S, n_my, ab, acc);
   float* base = out + ((int64_t)z * r + 128 * ti + 64 * wm + 4 * half) * r + 128 * tj + 64 * wn + l32;
 #pragma unroll
   for (int j = 0; j < 2; j++)
