@@ -138,7 +138,7 @@ constexpr int64_t SPMM_T_LONG = 256;    // columns longer than this get a whole 
 int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr);
 int launch_spmm_n_reduce(const dnpeff_csr* A, int r, float* N_nr);
 int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
-int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials);
+int launch_spsp(const dnpeff_csr* A, dnpeff_csr* B, float* partials);
 int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr);
 
 // Switches for experiments and for tests that force a code path.  Each has an environment
@@ -209,6 +209,9 @@ struct dnpeff_csr {
   int64_t* colptr = nullptr;
   int32_t* rowind = nullptr;
   float* tvals = nullptr;
+  // as the sparse factor of dnpeff_op_spsp_dense: per column 32 bytes holding its first four
+  // (row, value) pairs and, in the upper half of the first row word, its length
+  uint4* slots = nullptr;
   // work decomposition of A H^T: chunk_base[i] = chunks of rows before i
   int64_t* chunk_base = nullptr;
   int64_t n_chunks = 0;

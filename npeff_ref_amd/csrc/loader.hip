@@ -581,6 +581,7 @@ static void drop_derived(dnpeff_csr* A) {
   dfree(A->colptr); A->colptr = nullptr;
   dfree(A->rowind); A->rowind = nullptr;
   dfree(A->tvals); A->tvals = nullptr;
+  dfree(A->slots); A->slots = nullptr;
   dfree(A->chunk_base); A->chunk_base = nullptr; A->n_chunks = 0;
   dfree(A->long_cols); A->long_cols = nullptr; A->n_long = 0;
   dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
@@ -1534,6 +1535,7 @@ DN_API int dnpeff_csr_release(dnpeff_csr* A, int which) {
     dfree(A->colptr); A->colptr = nullptr;
     dfree(A->rowind); A->rowind = nullptr;
     dfree(A->tvals); A->tvals = nullptr;
+    dfree(A->slots); A->slots = nullptr;
     dfree(A->long_cols); A->long_cols = nullptr; A->n_long = 0;
   } else {
     DN_CHECK(false, "which must be 1 (row-major copy) or 2 (transposed copy)");

@@ -835,23 +835,41 @@ __global__ void __launch_bounds__(256)
 }
 
 // ---------------------------------------------------------------------------
-// partials[chunk, :] = sum over the chunk's entries (j, a) of a * B[:, j] for a
-// sparse B given by its transposed CSR (per column j: component ids and
-// values).  Each wave keeps its r running sums in LDS.  The entries of an A-row
-// chunk are applied strictly one after the other; within one entry the
-// components of column j are distinct, so lane k applies the k-th of them.
-// Every component therefore receives its additions in entry order.  Each lane
-// prefetches the first SPSP_PREFETCH components of "its" entry so that the
-// serial part touches registers and LDS only.
+// partials[chunk, :] = sum over the chunk's entries (j, a) of a * B[:, j] for a sparse B, a
+// lane per entry.  B's transposed copy (per column j: component ids and values) is condensed
+// into one 32-byte slot per column (its first four (component, value) pairs, the column's
+// length in the upper half of the first component word), so that an entry of A costs one
+// random sector instead of three dependent ones (column offsets, component ids, values); only
+// columns longer than four go on to the transposed arrays.  Each wave keeps its r running sums
+// in LDS and the lanes add into them with ds_add_f32: step k of a batch applies the k-th pair
+// of all 64 entries at once, and where two lanes meet in a component the LDS adds them one
+// after the other in lane order, the same way in every run.
 // ---------------------------------------------------------------------------
-constexpr int SPSP_PREFETCH = 4;
+__global__ void __launch_bounds__(256)
+    k_spsp_build_slots(int64_t n_cols, const int64_t* __restrict__ colptr, const int32_t* __restrict__ comp,
+                       const float* __restrict__ vals, uint4* __restrict__ slots) {
+  const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (j >= n_cols) return;
+  const int64_t q0 = colptr[j];
+  const int len = (int)(colptr[j + 1] - q0);
+  unsigned w[8];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    w[2 * k] = k < len ? (unsigned)comp[q0 + k] : 0u;
+    w[2 * k + 1] = k < len ? __float_as_uint(vals[q0 + k]) : 0u;
+  }
+  w[0] |= (unsigned)len << 16;
+  slots[2 * j] = make_uint4(w[0], w[1], w[2], w[3]);
+  slots[2 * j + 1] = make_uint4(w[4], w[5], w[6], w[7]);
+}
 
 template <int VPL>
 __global__ void __launch_bounds__(256)
-    k_spsp(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
-           const float* __restrict__ vals, const int64_t* __restrict__ chunk_base, int64_t n_rows,
-           int r, const int64_t* __restrict__ b_colptr, const int32_t* __restrict__ b_comp,
-           const float* __restrict__ b_vals, float* __restrict__ partials) {
+    k_spsp_slots(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
+                 const float* __restrict__ vals, const int64_t* __restrict__ chunk_base, int64_t n_rows,
+                 int r, const uint4* __restrict__ slots, const int64_t* __restrict__ b_colptr,
+                 const int32_t* __restrict__ b_comp, const float* __restrict__ b_vals,
+                 float* __restrict__ partials) {
   __shared__ float red[4][64 * VPL];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int64_t chunk = blockIdx.x;
@@ -869,54 +887,20 @@ __global__ void __launch_bounds__(256)
   for (int t = 0; t < VPL; t++) acc[lane + 64 * t] = 0.0f;
 
   for (int64_t e = w0; e < w1; e += 64) {
-    const int cnt = (w1 - e) < 64 ? (int)(w1 - e) : 64;
-    float my_a = 0.0f;
-    int64_t q0 = 0;
-    int len = 0;
-    int pc[SPSP_PREFETCH];
-    float pv[SPSP_PREFETCH];
-    if (lane < cnt) {
+    if (e + lane < w1) {
       const int32_t j = colind[e + lane];
-      my_a = vals[e + lane];
-      q0 = b_colptr[j];
-      len = (int)(b_colptr[j + 1] - q0);
-    }
-#pragma unroll
-    for (int k = 0; k < SPSP_PREFETCH; k++) {
-      pc[k] = 0;
-      pv[k] = 0.0f;
-      if (k < len) {
-        pc[k] = b_comp[q0 + k];
-        pv[k] = b_vals[q0 + k];
-      }
-    }
-    const int q0_lo = (int)(uint32_t)(q0 & 0xffffffffLL), q0_hi = (int)(q0 >> 32);
-    for (int u = 0; u < cnt; u++) {
-      const int len_u = bcast_i(len, u);
-      if (len_u == 0) continue;
-      const float a_u = bcast_f(my_a, u);
-      int c = bcast_i(pc[0], u);
-      float h = bcast_f(pv[0], u);
-#pragma unroll
-      for (int k = 1; k < SPSP_PREFETCH; k++) {
-        const int ck = bcast_i(pc[k], u);
-        const float hk = bcast_f(pv[k], u);
-        if (lane == k) {
-          c = ck;
-          h = hk;
-        }
-      }
-      const int first = len_u < SPSP_PREFETCH ? len_u : SPSP_PREFETCH;
-      if (lane < first) acc[c] = fmaf(a_u, h, acc[c]);
-      if (len_u > SPSP_PREFETCH) {
-        const int64_t q =
-            ((int64_t)bcast_i(q0_hi, u) << 32) | (int64_t)(uint32_t)bcast_i(q0_lo, u);
-        for (int k0 = SPSP_PREFETCH; k0 < len_u; k0 += 64) {
-          if (k0 + lane < len_u) {
-            const int cc = b_comp[q + k0 + lane];
-            const float hh = b_vals[q + k0 + lane];
-            acc[cc] = fmaf(a_u, hh, acc[cc]);
-          }
+      const float a = vals[e + lane];
+      const uint4 s0 = slots[2 * (int64_t)j];
+      const int len = (int)(s0.x >> 16);
+      if (len > 0) atomicAdd(&acc[s0.x & 0xffffu], a * __uint_as_float(s0.y));
+      if (len > 1) atomicAdd(&acc[s0.z], a * __uint_as_float(s0.w));
+      if (len > 2) {
+        const uint4 s1 = slots[2 * (int64_t)j + 1];
+        atomicAdd(&acc[s1.x], a * __uint_as_float(s1.y));
+        if (len > 3) atomicAdd(&acc[s1.z], a * __uint_as_float(s1.w));
+        if (len > 4) {
+          const int64_t q = b_colptr[j];
+          for (int k = 4; k < len; k++) atomicAdd(&acc[b_comp[q + k]], a * b_vals[q + k]);
         }
       }
     }
@@ -1243,7 +1227,7 @@ int launch_spmm_t_tile(const dnpeff_csr* A_full, int r, const float* W_nr, int64
   return launch_head_t_scatter(A_full, r, k0, k1, col0, T_tile);
 }
 
-int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials) {
+int launch_spsp(const dnpeff_csr* A, dnpeff_csr* B, float* partials) {
   const int r = (int)B->n_rows;
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   DN_CHECK(A->rowptr && A->chunk_base, "matrix has no row-major copy / work list");
@@ -1251,10 +1235,16 @@ int launch_spsp(const dnpeff_csr* A, const dnpeff_csr* B, float* partials) {
   DN_CHECK(A->n_cols == B->n_cols, "column counts differ (%lld vs %lld)", (long long)A->n_cols,
            (long long)B->n_cols);
   if (A->n_chunks == 0) return 0;
+  if (!B->slots && B->n_cols > 0) {
+    DN_TRY(dmalloc(&B->slots, 2 * B->n_cols));
+    hipLaunchKernelGGL(k_spsp_build_slots, dim3((unsigned)ceil_div(B->n_cols, 256)), dim3(256), 0, stream(),
+                       B->n_cols, B->colptr, B->rowind, B->tvals, B->slots);
+    DN_LAUNCH_CHECK();
+  }
   dim3 grid((unsigned)A->n_chunks), block(256);
-#define DN_SPSP(V)                                                                              \
-  hipLaunchKernelGGL((k_spsp<V>), grid, block, 0, stream(), A->rowptr, A->colind, A->vals,        \
-                     A->chunk_base, A->n_rows, r, B->colptr, B->rowind, B->tvals, partials)
+#define DN_SPSP(V)                                                                               \
+  hipLaunchKernelGGL((k_spsp_slots<V>), grid, block, 0, stream(), A->rowptr, A->colind, A->vals,   \
+                     A->chunk_base, A->n_rows, r, B->slots, B->colptr, B->rowind, B->tvals, partials)
   switch (vpl_for(r)) {
     case 1: DN_SPSP(1); break;
     case 2: DN_SPSP(2); break;
