@@ -211,7 +211,7 @@ static int launch_ptq(const float* P, int64_t ldp, int64_t K, const float* Q, in
 // way into LDS (three planes per operand, rows of 32 elements padded to 80 bytes: conflict-free
 // 16-byte reads), and a product is six MFMAs (split_bf16.hpp).  A workgroup of 4 waves owns a
 // 128 x 128 tile of C (wave (wm, wn): 64 x 64) and one slice of the contraction tiles of 32,
-// dealt round-robin; the next tile travels in registers while the MFMAs of the current one run.
+// dealt round-robin; the next two tiles travel in registers while the MFMAs of the current one run.
 // Per contraction tile a wave issues 48 MFMAs of 32 cycles and splits 32 elements (176 vector
 // instructions): 2240 SIMD cycles against 4096 for the 64 v_mfma_f32_32x32x2f32 of k_ptq.
 // Operands are zero-padded to whole tiles (rows to M_pad / N, the contraction to a multiple of
