@@ -12,6 +12,14 @@ namespace dn {
 
 typedef float acc16 __attribute__((ext_vector_type(16)));
 
+// n / den from the reciprocal (1 ulp) and one correction step: 5 vector instructions where the
+// IEEE division sequence takes 11.  For the epilogues of the split-operand updates, where
+// den = (X G) + eps is positive and normal; within 2 ulp of the quotient.
+__device__ __forceinline__ float mu_quotient(float n, float den) {
+  const float rc = __builtin_amdgcn_rcpf(den), q0 = n * rc;
+  return __builtin_fmaf(__builtin_fmaf(-den, q0, n), rc, q0);
+}
+
 // ---------------------------------------------------------------------------
 // F[i] *= num[i] / (den[i] + eps)      (divide first, then multiply)
 // ---------------------------------------------------------------------------
@@ -1030,7 +1038,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int v = 0; v < 16; v++) {
       const int64_t off = (32 * i + 8 * (v >> 2) + (v & 3)) * (int64_t)r + 32 * j + l32;
       const float d = acc[i][j][v];
-      const float q = n_[v] / (d + eps);
+      const float q = mu_quotient(n_[v], d + eps);
       tout[off] = x_[v] * q;
       if (WITH_D) tD[off] = d;
     }
@@ -1509,11 +1517,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       for (int v = 0; v < 16; v++) x[v] = xraw[(8 * (v >> 2) + 4 * half + (v & 3)) * XB_LDR + col];
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        // quotient from the reciprocal (1 ulp) and one correction step
-        const float den = a0[v] + eps, rc = __builtin_amdgcn_rcpf(den);
-        const float q0 = pn[v] * rc;
-        const float q = __builtin_fmaf(__builtin_fmaf(-den, q0, pn[v]), rc, q0);
-        const float o = x[v] * q;
+        const float o = x[v] * mu_quotient(pn[v], a0[v] + eps);
         pn[v] = o;
         (tout + (8 * (v >> 2) + (v & 3)) * r)[off0] = o;
       }
