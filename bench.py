@@ -285,7 +285,8 @@ def run_nmf(d, args, cfg):
     r = cfg["r"]
     cpu_rows = cpu_sample_rows(cfg) if args.cpu_steps > 0 else 0
     sample = prepare_cpu_sample(d, cfg, args.seed, cpu_rows) if 0 < cpu_rows < cfg["n"] else None
-    comparison = compare_decompositions(d, cfg, args.seed, r) if cfg.get("compare_rows") else None
+    comparison = (compare_decompositions(d, cfg, args.seed, r)
+                  if cfg.get("compare_rows") and not args.no_compare else None)
 
     free0, total = d.device_memory()
     t0 = time.perf_counter()
@@ -576,6 +577,8 @@ def main():
     ap.add_argument("--fp32-steps", type=int, default=2,
                     help="steps timed with the matrix products on the fp32 matrix cores (0 = skip)")
     ap.add_argument("--no-scipy", action="store_true")
+    ap.add_argument("--no-compare", action="store_true",
+                    help="configs[4]: skip the comparison of the A H^T decompositions on the first rows")
     args = ap.parse_args()
 
     if args.gpus != 1:

@@ -230,6 +230,8 @@ struct dnpeff_csr {
   int n_plain = 0, n_swept = 0;
   int32_t* panel_ids = nullptr;
   int* sweep_progress = nullptr;  // per-XCD counters of the sweep kernel (256 ints)
+  int32_t* sweep_perm = nullptr;  // the rows in the order the sweep kernel takes them
+  int64_t sweep_perm_key = 0;     // the launch shape that order was made for
   dn::panel_plan plan;
   int64_t* seg = nullptr;
   int32_t* pcol = nullptr;

@@ -564,6 +564,7 @@ static void drop_panels(dnpeff_csr* A) {
   dfree(A->panel_bounds); A->panel_bounds = nullptr;
   dfree(A->panel_ids); A->panel_ids = nullptr;
   dfree(A->sweep_progress); A->sweep_progress = nullptr;
+  dfree(A->sweep_perm); A->sweep_perm = nullptr; A->sweep_perm_key = 0;
   dfree(A->seg); A->seg = nullptr;
   dfree(A->pcol); A->pcol = nullptr;
   dfree(A->pval); A->pval = nullptr;

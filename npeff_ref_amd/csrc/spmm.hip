@@ -324,7 +324,11 @@ __global__ void __launch_bounds__(1024)
                    const int32_t* __restrict__ swept, int n_swept,
                    const int32_t* __restrict__ bounds_of, int slots, int slot0, int r, int stride,
                    const float* __restrict__ H, float* __restrict__ part,
-                   int* __restrict__ progress, int lag, int spin_max, int rows_wg) {
+                   int* __restrict__ progress, int lag, int spin_max, int rows_wg,
+                   const int32_t* __restrict__ perm) {
+  // [row0, row1) are positions in perm, the list of rows dealt so that every wave's rows hold
+  // about the same number of entries (rows of very different lengths would otherwise make the
+  // waves of a piece wait for the one with the longest rows).
   // r: components that this launch sums (4 LPR); stride: floats between two rows of H and of
   // the partial sums (the rank; r < stride for a launch on a slice of the components, whose H and
   // part pointers then start at the slice's first component)
@@ -337,7 +341,7 @@ __global__ void __launch_bounds__(1024)
   const int64_t q = blockIdx.x / SWEEP_XCDS, nq = gridDim.x / SWEEP_XCDS;
   int* const counter = progress + x * SWEEP_SYNC_STRIDE;
   const int n_pi = (n_swept - x + SWEEP_XCDS - 1) / SWEEP_XCDS;  // pieces of this XCD
-  auto row_of = [&](int i) { return row0 + ((int64_t)i * waves + wave) * nq + q; };
+  auto pos_of = [&](int i) { return row0 + ((int64_t)i * waves + wave) * nq + q; };
   // rows of this wave: those with i * waves + wave < rows_wg (at least two, at most 32)
   const int n_i = (rows_wg - wave + waves - 1) / waves;
 
@@ -348,8 +352,9 @@ __global__ void __launch_bounds__(1024)
   // (row_i, piece) segment of the current piece, lane 32 + i those of the next piece; a third
   // set (in the upper lanes of `st_*`) is on its way for the piece after that.  Lanes without a
   // row and pieces past the end hold empty segments.
-  const int64_t my_row = row_of(lane & 31);
-  const bool my_seg = (lane & 31) < n_i && my_row < row1;
+  const int64_t my_pos = pos_of(lane & 31);
+  const bool my_seg = (lane & 31) < n_i && my_pos < row1;
+  const int64_t my_row = my_seg ? perm[my_pos] : 0;
   auto load_off = [&](int pi, int64_t& s0, int& len) {
     const bool ok = my_seg && pi < n_pi;
     const int piece = swept[x + SWEEP_XCDS * (pi < n_pi ? pi : 0)];
@@ -591,8 +596,9 @@ __global__ void __launch_bounds__(1024)
   }
 
   for (int i = 0; i < n_i; i++) {
-    const int64_t row = row_of(i);
-    if (row < row1) {
+    const int64_t pos = pos_of(i);
+    if (pos < row1) {
+      const int64_t row = perm[pos];
       const float* src = sums + (size_t)(i * waves + wave) * r;
       float* dst = part + (row * slots + slot0 + x) * stride;
       for (int c = lane; c < r; c += 64) dst[c] = src[c];
@@ -999,7 +1005,55 @@ constexpr int SWEEP_REGISTER_BUDGET = 448;
 
 using sweep_kernel_t = void (*)(const int64_t*, const int32_t*, const float*, int64_t, int64_t, int,
                                 const int32_t*, int, const int32_t*, int, int, int, int, const float*,
-                                float*, int*, int, int, int);
+                                float*, int*, int, int, int, const int32_t*);
+
+__global__ void __launch_bounds__(256)
+    k_sweep_row_entries(const int64_t* __restrict__ seg, int64_t n_rows, int P, int64_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n_rows) out[i] = seg[i * (P + 1) + P] - seg[i * (P + 1)];
+}
+
+// The order in which the sweep kernel takes the rows: longest first, pass p takes every
+// n_pass-th of them, and within a pass the rows go to the (workgroup, wave) slots back and forth
+// (the slots of round i are the positions i * slots ... (i + 1) * slots - 1), so that the sums of
+// the slots' row lengths come out close.  pass_start[p] = first position of pass p.
+static int sweep_row_order(const dnpeff_csr* A, const sweep_shape& sh, std::vector<int64_t>& pass_start) {
+  dnpeff_csr* M = const_cast<dnpeff_csr*>(A);
+  const int64_t n = A->n_rows;
+  const int64_t slots = (int64_t)sh.waves * (sh.wgs / SWEEP_XCDS);
+  const int64_t key = (sh.n_pass << 32) ^ (slots << 8) ^ n;
+  pass_start.assign(sh.n_pass + 1, 0);
+  for (int64_t p = 0; p < sh.n_pass; p++)
+    pass_start[p + 1] = pass_start[p] + (n - p + sh.n_pass - 1) / sh.n_pass;
+  if (M->sweep_perm && M->sweep_perm_key == key) return 0;
+  DN_HIP(hipStreamSynchronize(stream()));
+  dfree(M->sweep_perm);
+  M->sweep_perm = nullptr;
+  dbuf<int64_t> counts;
+  DN_TRY(counts.alloc(n));
+  hipLaunchKernelGGL(k_sweep_row_entries, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream(), A->seg, n,
+                     A->n_panels, counts.p);
+  DN_LAUNCH_CHECK();
+  std::vector<int64_t> h(n);
+  DN_HIP(hipMemcpy(h.data(), counts.p, sizeof(int64_t) * n, hipMemcpyDeviceToHost));
+  std::vector<int32_t> order(n), perm(n);
+  for (int64_t i = 0; i < n; i++) order[i] = (int32_t)i;
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return h[a] > h[b]; });
+  for (int64_t p = 0; p < sh.n_pass; p++) {
+    const int64_t count = pass_start[p + 1] - pass_start[p];
+    for (int64_t t = 0; t < count; t++) {
+      const int64_t round = t / slots, first = round * slots;
+      const int64_t in_round = count - first < slots ? count - first : slots;
+      int64_t sl = t - first;
+      if (round & 1) sl = in_round - 1 - sl;
+      perm[pass_start[p] + first + sl] = order[p + t * sh.n_pass];
+    }
+  }
+  DN_TRY(dmalloc(&M->sweep_perm, n));
+  DN_HIP(hipMemcpy(M->sweep_perm, perm.data(), sizeof(int32_t) * n, hipMemcpyHostToDevice));
+  M->sweep_perm_key = key;
+  return 0;
+}
 
 // Ranks above 256 are swept in slices of 256 (or 128) components: one set of launches per slice,
 // each with its slice of every row of H pinned in the L2s and its own running sums.
@@ -1039,20 +1093,22 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
             kernel_regs[variant], (long long)sh.wgs, sh.waves, sh.rows_wg, (long long)sh.n_pass,
             (long long)sh.rows_per_pass, r / w, w);
   }
+  std::vector<int64_t> pass_start;
+  DN_TRY(sweep_row_order(A, sh, pass_start));
   const int32_t* swept = A->panel_ids + A->n_plain;
   int lag = (int)tuning().sweep_lag, spin_max = (int)tuning().sweep_spin;
   if (lag < 0) lag = 0;
   const size_t lds = sizeof(float) * (size_t)sh.rows_wg * w;
   for (int slice = 0; slice < r / w; slice++)
     for (int64_t pass = 0; pass < sh.n_pass; pass++) {
-      const int64_t row0 = pass * sh.rows_per_pass;
-      const int64_t row1 = row0 + sh.rows_per_pass < A->n_rows ? row0 + sh.rows_per_pass : A->n_rows;
+      const int64_t row0 = pass_start[pass], row1 = pass_start[pass + 1];
       hipLaunchKernelGGL(k_sweep_clear, dim3(1), dim3(SWEEP_XCDS * SWEEP_SYNC_STRIDE), 0, stream(),
                          A->sweep_progress);
       hipLaunchKernelGGL(kernel, dim3((unsigned)sh.wgs), dim3(64 * sh.waves), lds, stream(), A->seg,
                          A->pcol, A->pval, row0, row1, A->n_panels, swept, A->n_swept,
                          A->panel_bounds, slots, A->n_plain, w, r, H_mr + slice * w,
-                         A->partials + slice * w, A->sweep_progress, lag, spin_max, sh.rows_wg);
+                         A->partials + slice * w, A->sweep_progress, lag, spin_max, sh.rows_wg,
+                         A->sweep_perm);
       DN_LAUNCH_CHECK();
     }
   return 0;
