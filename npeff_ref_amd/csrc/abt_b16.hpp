@@ -75,7 +75,10 @@ struct AbtOperand {
 // exactly: past the last tile they fetch the last one again.  The sources must be readable for
 // whole tiles (zero padding, or rows clamped by the caller's pointer arithmetic); with A_KN /
 // B_KN the source and its leading dimension must be 16-byte aligned.
-template <bool A_KN, bool B_KN, int STAGES = 1>
+// SAME_AB: B is A (a diagonal tile of X^T X): the tile is fetched, split and stored once and both
+// operands are read from A's planes (a compile-time switch: a branch around the loads of B would
+// cost the exact waits).
+template <bool A_KN, bool B_KN, int STAGES = 1, bool SAME_AB = false>
 __device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, int64_t lda,
                                              const float* __restrict__ b_src, int64_t ldb,
                                              int64_t first, int64_t stride, int64_t n_tiles,
@@ -89,14 +92,14 @@ __device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, in
   auto fetch = [&](int s, int64_t t) {
     const int64_t k0 = (first + (t < n_tiles ? t : n_tiles - 1) * stride) * ABT_KB;
     oa[s].fetch(a_src, lda, k0);
-    ob[s].fetch(b_src, ldb, k0);
+    if constexpr (!SAME_AB) ob[s].fetch(b_src, ldb, k0);
   };
   auto commit = [&](int s) {
     oa[s].commit(ab);
-    ob[s].commit(ab + 3 * ABT_PLANE);
+    if constexpr (!SAME_AB) ob[s].commit(ab + 3 * ABT_PLANE);
   };
   const unsigned char* a_row = ab + (64 * wm + l32) * ABT_LD + 16 * half;
-  const unsigned char* b_row = ab + 3 * ABT_PLANE + (64 * wn + l32) * ABT_LD + 16 * half;
+  const unsigned char* b_row = ab + (SAME_AB ? 0 : 3 * ABT_PLANE) + (64 * wn + l32) * ABT_LD + 16 * half;
   auto mfma_tile = [&]() {
 #pragma unroll
     for (int st = 0; st < 2; st++) {

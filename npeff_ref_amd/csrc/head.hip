@@ -337,19 +337,41 @@ static int64_t gram_tiles_slices(int64_t rows, int r) {
   return s < 1 ? 1 : s;
 }
 
-int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
-  return (gram_tiles_slices(rows, r) + 1) * (int64_t)r * r;
+// The split-operand kernel runs the diagonal tile pairs and the others as two launches (a
+// diagonal pair fetches and splits one tile, not two), each with the slices that fill the 2
+// workgroup slots per CU once.
+static void gram_b16_slices(int64_t rows, int r, int64_t* s_diag, int64_t* s_off) {
+  const int64_t t = r / 128, slots = 2 * (int64_t)n_cus(), k_tiles = rows / 32;
+  int64_t d = slots / t, o = t > 1 ? slots / (t * (t - 1) / 2) : 0;
+  if (d < 1) d = 1;
+  if (t > 1 && o < 1) o = 1;
+  if (d > k_tiles) d = k_tiles;
+  if (o > k_tiles) o = k_tiles;
+  *s_diag = d < 1 ? 1 : d;
+  *s_off = t > 1 ? (o < 1 ? 1 : o) : 0;
 }
 
+int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
+  int64_t d, o;
+  gram_b16_slices(rows, r, &d, &o);
+  const int64_t s = std::max(gram_tiles_slices(rows, r), std::max(d, o));
+  return (s + 1) * (int64_t)r * r;
+}
+
+// Diagonal tiles hold s_diag slices, the others s_off, and slice number `extra` (if >= 0) holds
+// one more term of every tile (the last rows, from the fp32 kernel).
 __global__ void __launch_bounds__(256)
-    k_gram_tiles_reduce(const float* __restrict__ ws, int64_t slices, int r, float* __restrict__ G) {
+    k_gram_tiles_reduce(const float* __restrict__ ws, int64_t s_diag, int64_t s_off, int64_t extra, int r,
+                        float* __restrict__ G) {
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= r * r) return;
   const int a = e / r, b = e % r;
   if ((a >> 7) > (b >> 7) || ((a >> 7) == (b >> 7) && a > b)) return;  // upper triangle only
   double s = 0.0;
   const int64_t stride = (int64_t)r * r;
+  const int64_t slices = (a >> 7) == (b >> 7) ? s_diag : s_off;
   for (int64_t sl = 0; sl < slices; sl++) s += (double)ws[sl * stride + e];
+  if (extra >= 0) s += (double)ws[extra * stride + e];
   G[(int64_t)a * r + b] = (float)s;
   G[(int64_t)b * r + a] = (float)s;
 }
@@ -357,6 +379,9 @@ __global__ void __launch_bounds__(256)
 // The same on the bf16 matrix cores with split operands (abt_b16.hpp): both operand tiles are
 // column tiles of X, read with the contraction index (the rows of X) slow.  Whole contraction
 // tiles of 32 rows only; the caller adds the last rows.
+// DIAG: grid.x numbers the diagonal tiles; otherwise the tile pairs (ti < tj) row by row: every
+// workgroup of the grid works.
+template <bool DIAG>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_gram_tiles_b16(const float* __restrict__ X, int64_t k_tiles, int r, int n_tiles_side,
                      float* __restrict__ out) {
@@ -364,14 +389,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
-  // grid.x numbers the tile pairs (ti <= tj) row by row: every workgroup of the grid works
-  int p = blockIdx.x, row_len = n_tiles_side, ti = 0;
-  while (p >= row_len) {
-    p -= row_len;
-    ti++;
-    row_len--;
+  int ti = blockIdx.x, tj = blockIdx.x;
+  if (!DIAG) {
+    int p = blockIdx.x, row_len = n_tiles_side - 1;
+    ti = 0;
+    while (p >= row_len) {
+      p -= row_len;
+      ti++;
+      row_len--;
+    }
+    tj = ti + 1 + p;
   }
-  const int tj = ti + p;
   const int64_t S = gridDim.z, z = blockIdx.z;
   const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
   acc16 acc[2][2];
@@ -381,7 +409,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-  abt_mainloop<true, true, ABT_STAGES_GRAM>(X + 128 * ti, r, X + 128 * tj, r, z, S, n_my, ab, acc);
+  abt_mainloop<true, true, ABT_STAGES_GRAM, DIAG>(X + 128 * ti, r, X + 128 * tj, r, z, S, n_my, ab, acc);
   float* base = out + ((int64_t)z * r + 128 * ti + 64 * wm + 4 * half) * r + 128 * tj + 64 * wn + l32;
 #pragma unroll
   for (int j = 0; j < 2; j++)
@@ -393,35 +421,38 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace) {
-  int64_t slices = gram_tiles_slices(rows, r);
   const int t = r / 128;
+  int64_t s_diag, s_off, extra = -1;
   if (use_split_bf16() && rows >= ABT_KB) {
     static bool attr_set = false;
     if (!attr_set) {
-      DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_tiles_b16),
+      DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_tiles_b16<true>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+      DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_tiles_b16<false>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
       attr_set = true;
     }
     // whole contraction tiles on the bf16 matrix cores, the last rows (fewer than 32) as one
     // more slice through the fp32 kernel
     const int64_t k_tiles = rows / ABT_KB, whole = k_tiles * ABT_KB;
-    int64_t s = slices - 1;
-    if (s < 1) s = 1;
-    if (s > k_tiles) s = k_tiles;
-    hipLaunchKernelGGL(k_gram_tiles_b16, dim3((unsigned)(t * (t + 1) / 2), 1, (unsigned)s), dim3(256),
-                       ABT_LDS, stream(), X, k_tiles, r, t, workspace);
+    gram_b16_slices(rows, r, &s_diag, &s_off);
+    hipLaunchKernelGGL(k_gram_tiles_b16<true>, dim3((unsigned)t, 1, (unsigned)s_diag), dim3(256), ABT_LDS,
+                       stream(), X, k_tiles, r, t, workspace);
+    if (t > 1)
+      hipLaunchKernelGGL(k_gram_tiles_b16<false>, dim3((unsigned)(t * (t - 1) / 2), 1, (unsigned)s_off),
+                         dim3(256), ABT_LDS, stream(), X, k_tiles, r, t, workspace);
     DN_LAUNCH_CHECK();
-    slices = s;
     if (whole < rows) {
+      extra = std::max(s_diag, s_off);
       DN_TRY(launch_ptq(X + whole * r, r, rows - whole, X + whole * r, r, r, r, 1,
-                        workspace + s * (int64_t)r * r, t));
-      slices = s + 1;
+                        workspace + extra * (int64_t)r * r, t));
     }
   } else {
-    DN_TRY(launch_ptq(X, r, rows, X, r, r, r, slices, workspace, t));
+    s_diag = s_off = gram_tiles_slices(rows, r);
+    DN_TRY(launch_ptq(X, r, rows, X, r, r, r, s_diag, workspace, t));
   }
   hipLaunchKernelGGL(k_gram_tiles_reduce, dim3((unsigned)ceil_div((int64_t)r * r, 256)), dim3(256), 0,
-                     stream(), workspace, slices, r, G);
+                     stream(), workspace, s_diag, s_off, extra, r, G);
   DN_LAUNCH_CHECK();
   return 0;
 }
