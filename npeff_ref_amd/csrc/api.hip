@@ -152,7 +152,7 @@ static double product_overhead_bytes(const dnpeff_csr* A, int rank) {
 // Splits off the dense head when the products can use it: rank a multiple of 4 and at least 64
 // (below that a column of the dense block costs more than its entries do as gathers), enough
 // rows for the fill fraction to mean something.  A column goes to the head when at least 1/16 of
-// the rows hold it (dense_fill switch; 0 = never split); the fraction is doubled until the dense
+// the rows hold it (dense_fill switch; 0 = never split); the fraction is raised until the dense
 // blocks and both sparse copies of the rest fit the memory left beside the factors.  *tiled
 // receives whether the H update must run on column tiles for everything to fit.
 static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {

@@ -1166,7 +1166,8 @@ int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_block
   if (thr < 1) thr = 1;
   head_choice best = *out;  // "no head"
   bool have_fit = false;
-  for (; thr <= n && thr <= (int64_t)INT32_MAX; thr *= 2) {
+  // candidates a fifth apart (a doubled threshold can leave a quarter of the budget unused)
+  for (; thr <= n && thr <= (int64_t)INT32_MAX; thr = std::max(thr + 1, thr + thr / 5)) {
     int32_t n_d = 0;
     unsigned long long z_head = 0;
     DN_TRY(scan_keep_mask(count, (int)thr, m, pos));
