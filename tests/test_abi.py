@@ -140,6 +140,12 @@ def test_bench_work_model_and_sample_sizes():
     assert b == 12 * m * r + 4 * r * r and f == 2 * m * r * r and split
     assert bench.cpu_sample_rows(bench.CONFIGS["c1"]) == 10_000
     assert 256 <= bench.cpu_sample_rows(bench.CONFIGS["c3"]) <= 1024
-    assert bench.traffic_from_profile("c3", "spmm_n")[0] == pytest.approx(9.40e11)
+    # the value is whatever the committed counter summary holds (it changes with every refresh of
+    # the profile): parse the file here, independently, and compare
+    import os, re
+    path = os.path.join(bench.ROOT, "profiles", "nmf_c3_hbm_traffic.md")
+    held = [float(x) for x in re.findall(r"traffic_bytes\s+spmm_n\s+([0-9.eE+]+)", open(path).read())]
+    got, src = bench.traffic_from_profile("c3", "spmm_n")
+    assert held and got == held[0] and got > 8 * z and src == "profiles/nmf_c3_hbm_traffic.md"
     assert bench.traffic_from_profile("c3", "no_such_class") == (None, None)
     assert bench.traffic_from_profile("c0", "spmm_n") == (None, None)
