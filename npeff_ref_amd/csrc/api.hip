@@ -169,7 +169,7 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
     if (S0->colind) avail += 8.0 * (double)S0->nnz;
   }
   if (S0->colptr) avail += 8.0 * (double)S0->nnz;
-  if (S0->pcol) avail += 8.0 * (double)S0->nnz;
+  if (S0->pcol || S0->nl.pairs) avail += 8.0 * (double)S0->nnz;
   avail -= product_overhead_bytes(A, rank);
   const double budget_full = avail - factor_bytes(A->n_rows, A->n_cols, rank, false);
   const double budget_tiled = avail - factor_bytes(A->n_rows, A->n_cols, rank, true);

@@ -159,6 +159,11 @@ struct tuning_t {
   double h_tile_mb = 768.0;        // size of a column tile of the tiled H update, MiB of the factor
   double tiled_h = -1.0;           // tiled H update: 1 = always, 0 = never, -1 = when the full-size buffer does not fit
   double topk_fast_cap = -1.0;     // top-k: candidate list length that ends the histogram passes (-1 = default)
+  double n_lists = -1.0;           // A H^T from slot lists on component slices: 1 = always, 0 = never, -1 = by policy
+  double t_lists = -1.0;           // A^T W in column blocks on component slices: 1 / 0 / -1 likewise
+  double nl_piece_cols = 16384.0;  // columns per piece of the slot lists
+  double nl_lag = 1.0;             // pieces the workgroups of an XCD may be apart
+  double nl_flush = 64.0;          // batches of 64 entries between two moves of a slot's LDS sums into registers
   double verbose = 0.0;
 };
 tuning_t& tuning();
@@ -192,6 +197,28 @@ struct panel_plan {
   bool operator==(const panel_plan& o) const {
     return coarse == o.coarse && sweep_cols == o.sweep_cols && sweep_min == o.sweep_min;
   }
+};
+
+// Slot lists of A H^T on component slices (lists.hip): the entries of the sparse part as one
+// stream of (local row, local column, value) per wave slot, ordered by column piece.
+struct slot_lists {
+  int piece_cols = 0, n_pieces = 0, n_parts = 0, rpw = 0;
+  int64_t n_batches = 0;
+  uint2* pairs = nullptr;         // [n_batches + 8][64]
+  int64_t* slot_base = nullptr;   // [n_slots + 1] first batch of each slot
+  uint32_t* off = nullptr;        // [n_slots][n_pieces + 1] batches of the slot before piece p
+  int32_t* slot_rows = nullptr;   // [n_slots][rpw] row of each local row, -1 = none
+  int32_t* row_slot = nullptr;    // [n_rows] slot * 128 + local row
+  int* progress = nullptr;        // progress counters of the XCDs
+  std::vector<int32_t> h_row_slot;
+  std::vector<int64_t> h_slot_base;
+};
+
+// Column blocks of A^T W on component slices (lists.hip): cols[b] = first column of block b.
+struct col_blocks {
+  int32_t* cols = nullptr;  // [n_blocks + 1]
+  int64_t n_blocks = 0;
+  std::vector<int64_t> h_first;  // first block of every aligned group of 64 columns
 };
 
 }  // namespace dn
@@ -238,6 +265,8 @@ struct dnpeff_csr {
   float* pval = nullptr;
   // after dnpeff_csr_split_dense_head: the dense block and the matrix of the remaining entries
   // (same shape, owned), which carries the derived structures the products use
+  dn::slot_lists nl;
+  dn::col_blocks tb;
   dn::dense_head head;
   dnpeff_csr* tail = nullptr;
   // host copies of head.cols and long_cols (ascending), made when a product runs on column tiles
@@ -292,6 +321,19 @@ int csr_tile_lists(dnpeff_csr* A);
 inline bool has_row_major(const dnpeff_csr* A) {
   return A->rowptr != nullptr && (A->nnz == 0 || (A->colind != nullptr && A->vals != nullptr));
 }
+// lists.hip
+bool nlists_supported(const dnpeff_csr* S, int r);
+int nlists_build(dnpeff_csr* S, int r);
+void nlists_drop(dnpeff_csr* S);
+int launch_spmm_n_lists(const dnpeff_csr* S, int r, const float* H_mr, float* part);
+int nlists_get_row(const dnpeff_csr* S, int64_t row, std::vector<int32_t>& cols, std::vector<float>& vals);
+bool tlists_supported(const dnpeff_csr* S, int r);
+int tblocks_build(dnpeff_csr* S);
+void tblocks_drop(dnpeff_csr* S);
+int launch_spmm_t_lists(const dnpeff_csr* S, int r, const float* W_nr, float* T, int64_t col0, int64_t col1);
+// Whether the products of the sparse part S at rank r run from the slot lists / column blocks.
+bool use_nlists(const dnpeff_csr* S, int r);
+bool use_tlists(const dnpeff_csr* S, int r);
 struct head_choice {
   int64_t thr = 0;   // columns with at least thr entries form the head (0 = no head)
   int64_t n_d = 0;

@@ -61,6 +61,9 @@ static const tuning_entry g_tuning_table[] = {
     {"split_bf16", &tuning_t::split_bf16},       {"fused_gram", &tuning_t::fused_gram},
     {"h_tile_mb", &tuning_t::h_tile_mb},         {"tiled_h", &tuning_t::tiled_h},
     {"topk_fast_cap", &tuning_t::topk_fast_cap}, {"verbose", &tuning_t::verbose},
+    {"n_lists", &tuning_t::n_lists},             {"t_lists", &tuning_t::t_lists},
+    {"nl_piece_cols", &tuning_t::nl_piece_cols}, {"nl_lag", &tuning_t::nl_lag},
+    {"nl_flush", &tuning_t::nl_flush},
 };
 
 static tuning_t tuning_from_env() {
@@ -579,6 +582,8 @@ static void drop_derived(dnpeff_csr* A) {
   A->h_lists_valid = false;
   drop_head(A);
   drop_panels(A);
+  nlists_drop(A);
+  tblocks_drop(A);
   dfree(A->colptr); A->colptr = nullptr;
   dfree(A->rowind); A->rowind = nullptr;
   dfree(A->tvals); A->tvals = nullptr;
@@ -728,10 +733,34 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   return plan;
 }
 
+// The products of a sparse part run on component slices (lists.hip) when the switches n_lists /
+// t_lists say so (1) or leave it to the policy (-1): rank a multiple of 32, workgroups dealt to the
+// XCDs round-robin, and a factor too large for the caches (A H^T) / a slice of W that an L2 holds
+// (A^T W).
+bool use_nlists(const dnpeff_csr* S, int r) {
+  const double sw = tuning().n_lists;
+  if (sw == 0.0 || !nlists_supported(S, r)) return false;
+  if (sw > 0.0) return true;
+  return xcd_round_robin() && 4.0 * (double)S->n_cols * r >= 512e6 && S->n_rows >= 2048 && r >= 128;
+}
+bool use_tlists(const dnpeff_csr* S, int r) {
+  const double sw = tuning().t_lists;
+  if (sw == 0.0 || !tlists_supported(S, r)) return false;
+  if (sw > 0.0) return true;
+  return xcd_round_robin() && 128.0 * (double)S->n_rows <= 3.2e6 && 4.0 * (double)S->n_rows * r > 6.0e6;
+}
+
 int csr_ensure_products(dnpeff_csr* A, int r) {
   dnpeff_csr* S = sparse_part(A);
   DN_TRY(dnpeff_csr_build_transpose(S));
-  DN_TRY(csr_set_panels(S, panel_policy(S, r)));
+  if (use_nlists(S, r)) {
+    DN_TRY(csr_set_panels(S, panel_plan()));
+    DN_TRY(nlists_build(S, r));
+  } else {
+    nlists_drop(S);
+    DN_TRY(csr_set_panels(S, panel_policy(S, r)));
+  }
+  if (use_tlists(S, r)) DN_TRY(tblocks_build(S));
   DN_TRY(csr_ensure_partials(S, r));
   return head_ensure_workspace(A, r);
 }
@@ -745,7 +774,7 @@ int csr_consume_for_products(dnpeff_csr* A) {
     dfree(A->chunk_base); A->chunk_base = nullptr; A->n_chunks = 0;
     dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
   }
-  if (S->n_panels > 0 && S->nnz > 0) {  // A H^T reads the regrouped copy
+  if ((S->n_panels > 0 || S->nl.pairs) && S->nnz > 0) {  // A H^T reads the regrouped copy / the slot lists
     DN_TRY(csr_ensure_chunks(S));  // (sizes the partial sums; needs the row offsets only)
     dfree(S->colind); S->colind = nullptr;
     dfree(S->vals); S->vals = nullptr;
@@ -774,6 +803,7 @@ int csr_ensure_partials(dnpeff_csr* A, int r) {
   int64_t need = A->n_chunks * (int64_t)r;
   if (A->n_panels > 0 && A->n_rows * panel_slots(A) * (int64_t)r > need)
     need = A->n_rows * panel_slots(A) * (int64_t)r;
+  if (A->nl.pairs && A->n_rows * (int64_t)r > need) need = A->n_rows * (int64_t)r;
   if (need <= A->partials_floats && A->partials) return 0;
   dfree(A->partials);
   A->partials = nullptr;
@@ -1444,7 +1474,15 @@ DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* 
   DN_HIP(hipMemcpy(e, S->rowptr + row, sizeof(e), hipMemcpyDeviceToHost));
   const int32_t* src_c = S->colind ? S->colind : S->pcol;
   const float* src_v = S->vals ? S->vals : S->pval;
-  DN_CHECK(e[1] == e[0] || (src_c && src_v), "matrix holds no row-major copy of its sparse part");
+  std::vector<int32_t> list_cols;
+  std::vector<float> list_vals;
+  if (!(src_c && src_v) && S->nl.pairs) {  // the sparse part is held as slot lists
+    DN_TRY(nlists_get_row(S, row, list_cols, list_vals));
+    DN_CHECK((int64_t)list_cols.size() == e[1] - e[0], "slot lists hold %lld entries of row %lld, not %lld",
+             (long long)list_cols.size(), (long long)row, (long long)(e[1] - e[0]));
+  } else {
+    DN_CHECK(e[1] == e[0] || (src_c && src_v), "matrix holds no row-major copy of its sparse part");
+  }
   int64_t got = e[1] - e[0];
   std::vector<float> head_row;
   std::vector<int32_t> head_cols;
@@ -1472,7 +1510,10 @@ DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* 
       cols[w] = head_cols[k];
       vals[w++] = head_row[k];
     }
-  if (e[1] > e[0]) {
+  if (!list_cols.empty()) {
+    memcpy(cols + w, list_cols.data(), sizeof(int32_t) * list_cols.size());
+    memcpy(vals + w, list_vals.data(), sizeof(float) * list_vals.size());
+  } else if (e[1] > e[0]) {
     DN_HIP(hipMemcpy(cols + w, src_c + e[0], sizeof(int32_t) * (e[1] - e[0]), hipMemcpyDeviceToHost));
     DN_HIP(hipMemcpy(vals + w, src_v + e[0], sizeof(float) * (e[1] - e[0]), hipMemcpyDeviceToHost));
   }

@@ -1119,6 +1119,10 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
   DN_TRY(launch_head_n(A_full, r, H_mr));
   const dnpeff_csr* A = sparse_part(A_full);
   float* partials = A->partials;
+  if (A->nl.pairs && use_nlists(A, r)) {
+    DN_CHECK(partials && A->partials_floats >= A->n_rows * (int64_t)r, "partial sums too small");
+    return launch_spmm_n_lists(A, r, H_mr, partials);
+  }
   if (A->n_panels > 0) {
     DN_CHECK(A->seg && A->pcol && A->panel_ids && partials, "matrix has no panel work list");
     const bool aligned = ((uintptr_t)H_mr % 16) == 0;
@@ -1155,12 +1159,13 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
 
 int launch_spmm_n_reduce(const dnpeff_csr* A_full, int r, float* N_nr) {
   const dnpeff_csr* A = sparse_part(A_full);
-  if (A->n_panels > 0) {
+  const bool lists = A->nl.pairs && use_nlists(A, r);  // one set of sums, no panels
+  if (lists || A->n_panels > 0) {
     if (A->n_rows > 0) {
       int64_t wgs = ceil_div(A->n_rows * r, 256);
       if (wgs > (1 << 20)) wgs = 1 << 20;
       hipLaunchKernelGGL(k_panel_reduce, dim3((unsigned)wgs), dim3(256), 0, stream(), A->partials,
-                         A->n_rows, (int)panel_slots(A), r, N_nr);
+                         A->n_rows, lists ? 1 : (int)panel_slots(A), r, N_nr);
       DN_LAUNCH_CHECK();
     }
   } else {
@@ -1203,6 +1208,8 @@ static int launch_spmm_t_sparse(const dnpeff_csr* A, int r, const float* W_nr, f
   if (m <= 0) return 0;
   const int64_t* colptr = A->colptr + col0;
   const bool aligned = ((uintptr_t)T % 16) == 0 && ((uintptr_t)W_nr % 16) == 0;
+  if (A->tb.cols && aligned && col0 % 64 == 0 && (col1 % 64 == 0 || col1 == A->n_cols) && use_tlists(A, r))
+    return launch_spmm_t_lists(A, r, W_nr, T, col0, col1);
   const int n_slices = (aligned && r % 4 == 0) ? spmm_t_slices(A->n_rows, r) : 1;
   const int width = r / n_slices;
   // one wave per (column, slice); a launch holds at most 2^32 threads, so beyond 2^23 workgroups
