@@ -159,11 +159,12 @@ struct tuning_t {
   double h_tile_mb = 768.0;        // size of a column tile of the tiled H update, MiB of the factor
   double tiled_h = -1.0;           // tiled H update: 1 = always, 0 = never, -1 = when the full-size buffer does not fit
   double topk_fast_cap = -1.0;     // top-k: candidate list length that ends the histogram passes (-1 = default)
-  double n_lists = -1.0;           // A H^T from slot lists on component slices: 1 = always, 0 = never, -1 = by policy
-  double t_lists = -1.0;           // A^T W in column blocks on component slices: 1 / 0 / -1 likewise
+  double n_lists = 0.0;            // A H^T from slot lists on component slices (1 = on)
+  double t_lists = 0.0;            // A^T W in column blocks on component slices (1 = on)
   double nl_piece_cols = 16384.0;  // columns per piece of the slot lists
   double nl_lag = 1.0;             // pieces the workgroups of an XCD may be apart
-  double nl_flush = 64.0;          // batches of 64 entries between two moves of a slot's LDS sums into registers
+  double nl_wgs = 64.0;            // workgroups of the slot-list kernel per XCD (two per CU)
+  double nl_spin = 50000.0;        // polls (about 1 us each) before a workgroup of the slot-list kernel stops waiting
   double verbose = 0.0;
 };
 tuning_t& tuning();
@@ -202,7 +203,7 @@ struct panel_plan {
 // Slot lists of A H^T on component slices (lists.hip): the entries of the sparse part as one
 // stream of (local row, local column, value) per wave slot, ordered by column piece.
 struct slot_lists {
-  int piece_cols = 0, n_pieces = 0, n_parts = 0, rpw = 0;
+  int piece_cols = 0, n_pieces = 0, n_parts = 0, rpw = 0, wgs = 0;
   int64_t n_batches = 0;
   uint2* pairs = nullptr;         // [n_batches + 8][64]
   int64_t* slot_base = nullptr;   // [n_slots + 1] first batch of each slot

@@ -63,7 +63,7 @@ static const tuning_entry g_tuning_table[] = {
     {"topk_fast_cap", &tuning_t::topk_fast_cap}, {"verbose", &tuning_t::verbose},
     {"n_lists", &tuning_t::n_lists},             {"t_lists", &tuning_t::t_lists},
     {"nl_piece_cols", &tuning_t::nl_piece_cols}, {"nl_lag", &tuning_t::nl_lag},
-    {"nl_flush", &tuning_t::nl_flush},
+    {"nl_spin", &tuning_t::nl_spin},             {"nl_wgs", &tuning_t::nl_wgs},
 };
 
 static tuning_t tuning_from_env() {
@@ -733,21 +733,15 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
   return plan;
 }
 
-// The products of a sparse part run on component slices (lists.hip) when the switches n_lists /
-// t_lists say so (1) or leave it to the policy (-1): rank a multiple of 32, workgroups dealt to the
-// XCDs round-robin, and a factor too large for the caches (A H^T) / a slice of W that an L2 holds
-// (A^T W).
+// The products of a sparse part run on component slices (lists.hip) only when the switches
+// n_lists / t_lists ask for it (1): at the sizes measured they are slower than the panels, swept
+// pieces and 4-slice column kernel that the plan uses otherwise.  Needs a rank that is a multiple
+// of 32 and workgroups dealt to the XCDs round-robin.
 bool use_nlists(const dnpeff_csr* S, int r) {
-  const double sw = tuning().n_lists;
-  if (sw == 0.0 || !nlists_supported(S, r)) return false;
-  if (sw > 0.0) return true;
-  return xcd_round_robin() && 4.0 * (double)S->n_cols * r >= 512e6 && S->n_rows >= 2048 && r >= 128;
+  return tuning().n_lists > 0.0 && nlists_supported(S, r) && xcd_round_robin();
 }
 bool use_tlists(const dnpeff_csr* S, int r) {
-  const double sw = tuning().t_lists;
-  if (sw == 0.0 || !tlists_supported(S, r)) return false;
-  if (sw > 0.0) return true;
-  return xcd_round_robin() && 128.0 * (double)S->n_rows <= 3.2e6 && 4.0 * (double)S->n_rows * r > 6.0e6;
+  return tuning().t_lists > 0.0 && tlists_supported(S, r) && xcd_round_robin();
 }
 
 int csr_ensure_products(dnpeff_csr* A, int r) {

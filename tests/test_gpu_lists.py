@@ -28,7 +28,6 @@ def test_spmm_n_from_slot_lists(r, shape, piece_cols, tune):
     n, m, maxk = shape
     tune("n_lists", 1)
     tune("nl_piece_cols", piece_cols)
-    tune("nl_flush", 2)
     rng = np.random.default_rng(r + n)
     rp, ci, va = random_csr(rng, n, m, maxk, empty_rows={1, n - 1})
     A = d.Csr.from_host(rp, ci, va, m)
@@ -42,7 +41,7 @@ def test_spmm_n_from_slot_lists(r, shape, piece_cols, tune):
     d.op_spmm_n(A, r, dH, dN)
     assert np.array_equal(dN.numpy(), N)
     tune("nl_lag", 3)
-    tune("sweep_spin", 1)
+    tune("nl_spin", 1)
     d.op_spmm_n(A, r, dH, dN)
     assert np.array_equal(dN.numpy(), N)
     A.close()
