@@ -61,9 +61,25 @@ void* dnpeff_stream(void);
  * (cc/cuda_d_npeff/src/cuda/debugging/). */
 int dnpeff_device_memory(int64_t* free_bytes, int64_t* total_bytes);
 
+/* The byte table behind the memory plan of dnpeff_nmf_create, computable without a GPU (capacity
+ * planning, tests): for a matrix of n_rows x n_cols whose sparse part holds nnz_sparse entries
+ * and whose dense head holds n_dense columns, at the given rank, with the tiled (1) or full-size
+ * (0) H update, on a device of total_bytes; sweeps = 1 when A H^T has swept pieces (ranks 32, 64,
+ * 128, 256 and multiples of 128 above, on a device whose workgroups go to the XCDs round-robin).
+ * out[0..7] = factors and their workspaces, partial sums of A H^T, segment offsets, column/row
+ * offsets, reserve left free, both sparse copies, dense blocks of the head, workspace of the
+ * head's products; all in bytes, upper bounds from the rules that size the allocations.  The
+ * reference sizes its buffers inside the constructor
+ * (multi_mu_dense_factors_device_contexts1.h:128-200) and has no such call. */
+int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int64_t n_dense, int rank,
+                         int tiled, int sweeps, int64_t total_bytes, double* out);
+
 /* Switches for experiments and for tests that must reach a particular code path; no counterpart
  * in the reference.  Names: dense_fill, panels, sweep_bytes, sweep_min, sweep_waves, sweep_lag,
- * sweep_spin, spmm_t_slices, split_bf16, fused_gram, h_tile_mb, tiled_h, topk_fast_cap, verbose.
+ * sweep_spin, spmm_t_slices, split_bf16, fused_gram, h_tile_mb, tiled_h, topk_fast_cap, verbose,
+ * gram_beside (H^T H of the W update on a second stream beside A H^T), n_lists, t_lists (the sparse
+ * products on component slices of 32: slot lists / column blocks), nl_piece_cols, nl_lag, nl_spin,
+ * nl_wgs (their piece size, lock step and launch shape).
  * Each starts from the environment variable DNPEFF_<NAME IN CAPITALS> (read once, when the
  * library is first used) or its default; plans take the values when they are made
  * (dnpeff_nmf_create, the first product on a matrix).  dnpeff_tuning_reset() goes back to the

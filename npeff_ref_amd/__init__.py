@@ -30,6 +30,7 @@ from .binding import (  # noqa: F401
     sync,
     device_info,
     device_memory,
+    plan_estimate,
     tuning_set,
     tuning_get,
     tuning_reset,

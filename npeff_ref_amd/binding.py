@@ -48,6 +48,7 @@ SIGNATURES = {
     "dnpeff_device_memory": (C.c_int, [C.POINTER(_i64), C.POINTER(_i64)]),
     "dnpeff_tuning_set": (C.c_int, [C.c_char_p, _f64]),
     "dnpeff_tuning_get": (C.c_int, [C.c_char_p, C.POINTER(_f64)]),
+    "dnpeff_plan_estimate": (C.c_int, [_i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, _i64, C.POINTER(_f64)]),
     "dnpeff_tuning_reset": (C.c_int, []),
     "dnpeff_dev_malloc": (C.c_int, [_i64, _pp]),
     "dnpeff_dev_free": (C.c_int, [_p]),
@@ -169,6 +170,18 @@ def device_memory():
     f, t = _i64(0), _i64(0)
     _check(lib.dnpeff_device_memory(C.byref(f), C.byref(t)))
     return f.value, t.value
+
+
+PLAN_FIELDS = ("factors", "partials", "segments", "offsets", "reserve", "sparse_copies", "head_blocks",
+               "head_workspace")
+
+
+def plan_estimate(n_rows, n_cols, nnz_sparse, n_dense, rank, tiled, sweeps=True, total_bytes=309_220_868_096):
+    """The byte table of the memory plan (dnpeff_plan_estimate) as a dict; needs no GPU."""
+    out = (_f64 * 8)()
+    _check(lib.dnpeff_plan_estimate(n_rows, n_cols, nnz_sparse, n_dense, rank, int(bool(tiled)), int(bool(sweeps)),
+                                    total_bytes, out))
+    return dict(zip(PLAN_FIELDS, [float(x) for x in out]))
 
 
 def tuning_set(name: str, value: float):

@@ -2,6 +2,7 @@
 // run_nmf_on_pefs and the W-only learner of fit_coeffs_to_sparse_H.
 #include "dnpeff_internal.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <utility>
@@ -139,14 +140,52 @@ static double factor_bytes(int64_t n, int64_t m, int rank, bool tiled) {
          4.0 * (double)xg_mu_gram_workspace_floats(m);
 }
 
-// What the products' own buffers take besides the two sparse copies and the dense blocks: partial
-// sums of A H^T, segment offsets, column offsets, work lists, head workspace (upper estimates),
-// plus room that is left free.
-static double product_overhead_bytes(const dnpeff_csr* A, int rank) {
-  const double n = (double)A->n_rows, m = (double)A->n_cols;
-  double partials = 4.0 * rank * (double)A->nnz / (double)SPMM_N_CHUNK + 4.0 * rank * n;
-  if (partials < 3.2e9 && 4.0 * m * rank >= 512e6) partials = 3.2e9;
-  return partials + 8.0 * n * 3100.0 + 8.0 * m + 4.0 * m + 1.5e9 + 4.0e9;
+// What the products' own buffers take besides the two sparse copies (16 bytes per entry of the
+// sparse part), the dense blocks and the head's workspace, which the choice of the head prices
+// per candidate: upper bounds from the same rules that size the allocations.
+struct plan_table {
+  double factors = 0.0;   // W, its double buffer, A H^T, H (+ tile), A^T W (or its tile), Grams, workspaces
+  double partials = 0.0;  // partial sums of A H^T: per 2048-entry chunk, or per (row, plain panel / XCD)
+  double segments = 0.0;  // offsets of the (row, panel) segments
+  double offsets = 0.0;   // column offsets, long-column list, row offsets and chunk counts
+  double reserve = 0.0;   // left free (1/64 of the device, at least 1 GiB): allocation granularity, code objects, the runtime's own
+  double total() const { return factors + partials + segments + offsets + reserve; }
+};
+
+static plan_table plan_overheads(int64_t n, int64_t m, int64_t nnz_sparse, int rank, bool tiled, bool sweeps,
+                                 double total_bytes) {
+  plan_table t;
+  t.factors = factor_bytes(n, m, rank, tiled);
+  const int64_t P = coarse_panels_for(n, m, rank, sweeps);
+  const double by_chunks = 4.0 * rank * ((double)nnz_sparse / (double)SPMM_N_CHUNK + (double)n);
+  const double by_panels = P > 0 ? 4.0 * rank * (double)n * (double)(P + SWEEP_XCDS) : 0.0;
+  t.partials = by_chunks > by_panels ? by_chunks : by_panels;
+  // (a coarse panel may be cut into swept pieces: up to max_panels() panels and pieces in all)
+  t.segments = P > 0 ? 8.0 * (double)n * (double)((sweeps ? max_panels() : P) + 1) : 0.0;
+  const double n_long = std::min((double)m, (double)nnz_sparse / (double)(SPMM_T_LONG + 1));
+  t.offsets = 8.0 * (double)(m + 1) + 4.0 * n_long + 2.0 * 8.0 * (double)(n + 1) + 2.0 * 8.0 * 64.0;
+  t.reserve = std::max(1073741824.0, total_bytes / 64.0);
+  return t;
+}
+
+// For tests and capacity planning without a GPU: the table above and, for a head of n_dense columns,
+// its blocks and workspace.  out[0..7] = factors, partials, segments, offsets, reserve, sparse
+// copies, head blocks, head workspace (bytes).
+DN_API int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int64_t n_dense, int rank,
+                                int tiled, int sweeps, int64_t total_bytes, double* out) {
+  clear_error();
+  DN_CHECK(out != nullptr, "out is NULL");
+  DN_CHECK(n_rows >= 0 && n_cols >= 0 && nnz_sparse >= 0 && n_dense >= 0 && n_dense <= n_cols,
+           "negative size");
+  DN_CHECK(rank >= 1 && rank <= 1024, "rank %d outside [1, 1024]", rank);
+  const plan_table t = plan_overheads(n_rows, n_cols, nnz_sparse, rank, tiled != 0, sweeps != 0, (double)total_bytes);
+  out[0] = t.factors; out[1] = t.partials; out[2] = t.segments; out[3] = t.offsets; out[4] = t.reserve;
+  out[5] = 16.0 * (double)nnz_sparse;
+  out[6] = n_dense ? 4.0 * head_blocks_for_rank(rank) * (double)(ceil_div(n_rows, 128) * 128) *
+                         (double)(ceil_div(n_dense, 128) * 128)
+                   : 0.0;
+  out[7] = 4.0 * (double)head_workspace_floats(n_rows, n_dense, rank);
+  return 0;
 }
 
 // Splits off the dense head when the products can use it: rank a multiple of 4 and at least 64
@@ -170,9 +209,11 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
   }
   if (S0->colptr) avail += 8.0 * (double)S0->nnz;
   if (S0->pcol || S0->nl.pairs) avail += 8.0 * (double)S0->nnz;
-  avail -= product_overhead_bytes(A, rank);
-  const double budget_full = avail - factor_bytes(A->n_rows, A->n_cols, rank, false);
-  const double budget_tiled = avail - factor_bytes(A->n_rows, A->n_cols, rank, true);
+  const bool sweeps = sweeps_for_rank(rank);
+  const plan_table t_full = plan_overheads(A->n_rows, A->n_cols, A->nnz, rank, false, sweeps, (double)total_b);
+  const plan_table t_tiled = plan_overheads(A->n_rows, A->n_cols, A->nnz, rank, true, sweeps, (double)total_b);
+  const double budget_full = avail - t_full.total();
+  const double budget_tiled = avail - t_tiled.total();
   const bool can_split = rank % 4 == 0 && rank >= 64 && A->n_rows >= 1024;
   double fill = tn.dense_fill;
   if (fill > 1.0) fill = 0.0;
@@ -180,7 +221,7 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
   if (A->tail) {
     if (rank % 4 == 0) {  // split by the caller (or an earlier handle): keep it
       const double foot = 4.0 * head_blocks_for_rank(rank) * (double)A->head.n_pad * (double)A->head.n_d_pad +
-                          16.0 * (double)S0->nnz;
+                          16.0 * (double)S0->nnz + 4.0 * (double)head_workspace_floats(A->n_rows, A->head.n_d, rank);
       if (tn.tiled_h < 0.0) *tiled = foot > budget_full;
       return 0;
     }
@@ -194,18 +235,23 @@ static int plan_matrix(dnpeff_csr* A, int rank, bool consume, bool* tiled) {
   }
   head_choice c;
   const int n_blocks = head_blocks_for_rank(rank);
-  DN_TRY(choose_dense_head(A, fill, *tiled ? budget_tiled : budget_full, n_blocks, &c));
+  DN_TRY(choose_dense_head(A, fill, *tiled ? budget_tiled : budget_full, n_blocks, rank, &c));
   if (!c.fits && tn.tiled_h < 0.0 && !*tiled) {
     *tiled = true;
-    DN_TRY(choose_dense_head(A, fill, budget_tiled, n_blocks, &c));
+    DN_TRY(choose_dense_head(A, fill, budget_tiled, n_blocks, rank, &c));
   }
-  if (tn.verbose != 0.0)
+  if (tn.verbose != 0.0) {
+    const plan_table& t = *tiled ? t_tiled : t_full;
     fprintf(stderr,
             "dnpeff: plan for rank %d: %.1f GB free, budget for the matrix %.1f GB (%s H update); dense "
-            "head of %lld columns (>= %lld entries), footprint %.1f GB%s\n",
+            "head of %lld columns (>= %lld entries), footprint %.1f GB%s\n"
+            "dnpeff: plan bytes: factors %.2f GB, partial sums %.2f GB, segment offsets %.2f GB, column "
+            "offsets %.2f GB, reserve %.2f GB\n",
             rank, (double)free_b / 1e9, (*tiled ? budget_tiled : budget_full) / 1e9,
             *tiled ? "tiled" : "full-size", (long long)c.n_d, (long long)c.thr, c.footprint / 1e9,
-            c.fits ? "" : " (over budget)");
+            c.fits ? "" : " (over budget)", t.factors / 1e9, t.partials / 1e9, t.segments / 1e9,
+            t.offsets / 1e9, t.reserve / 1e9);
+  }
   if (c.thr == 0) return 0;  // no head (there is none to undo either)
   return split_dense_head_at(A, c.thr, nullptr);
 }
@@ -324,6 +370,17 @@ static int products_for(dnpeff_nmf* h) {
 DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
+  // H^T H and A H^T both only read H: with the gram_beside switch the Gram kernel (bound by
+  // instruction issue) runs on a second stream beside the head product and the plain panels of
+  // A H^T (bound by the fabric)
+  bool gram_done = false;
+  if (!h->nw_valid && !h->gh_valid && tuning().gram_beside != 0.0) {
+    DN_TRY(side_stream_begin());
+    int st = launch_gram(h->m, h->r, h->H, h->G, h->gram_ws);
+    DN_TRY(side_stream_end());
+    DN_TRY(st);
+    gram_done = true;
+  }
   if (!h->nw_valid) {  // a loss evaluation since the last H update has left A H^T in Nw
     DN_TRY(products_for(h));
     DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N));
@@ -335,7 +392,10 @@ DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
     h->nw_valid = true;
   }
   const float* Gh = h->GH;
-  if (!h->gh_valid) {
+  DN_TRY(side_stream_join());
+  if (gram_done) {
+    Gh = h->G;
+  } else if (!h->gh_valid) {
     DN_TRY(h->prof.begin(DNPEFF_K_GRAM_H));
     DN_TRY(launch_gram(h->m, h->r, h->H, h->G, h->gram_ws));
     DN_TRY(h->prof.end());

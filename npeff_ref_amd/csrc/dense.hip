@@ -79,7 +79,10 @@ static int gram_pairs(int r) {
 
 static bool gram_uses_tiles(int64_t rows, int r) { return r > 128 && r % 128 == 0 && rows >= 1024; }
 
+static int64_t gram_small_wgs(int64_t rows);
+
 int64_t gram_workspace_floats(int64_t rows, int r) {
+  if (r <= 32) return gram_small_wgs(rows) * 1024;  // one 32 x 32 block per workgroup of k_gram_small
   if (gram_uses_tiles(rows, r)) return gram_tiles_workspace_floats(rows, r);
   return gram_slices(rows) * (int64_t)gram_pairs(r) * 1024;
 }

@@ -21,6 +21,10 @@ void clear_error();
 hipStream_t stream();
 // Compute units of device 0.
 int n_cus();
+// A second stream for work that may run beside the library stream (see loader.hip).
+int side_stream_begin();
+int side_stream_end();
+int side_stream_join();
 
 }  // namespace dn
 
@@ -163,6 +167,7 @@ struct tuning_t {
   double t_lists = 0.0;            // A^T W in column blocks on component slices (1 = on)
   double nl_piece_cols = 16384.0;  // columns per piece of the slot lists
   double nl_lag = 1.0;             // pieces the workgroups of an XCD may be apart
+  double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
   double nl_wgs = 64.0;            // workgroups of the slot-list kernel per XCD (two per CU)
   double nl_spin = 50000.0;        // polls (about 1 us each) before a workgroup of the slot-list kernel stops waiting
   double verbose = 0.0;
@@ -227,6 +232,11 @@ struct col_blocks {
 struct dnpeff_csr {
   int64_t n_rows = 0, n_cols = 0, nnz = 0;
   int64_t full_dense_size = 0;
+  // ||A||_F^2 as first computed (from the row-major values, in their order); the loader calls that
+  // change entries clear it.  Kept so that a matrix whose arrays a context has consumed still
+  // gives later contexts the same number.
+  double sq_norm = 0.0;
+  bool sq_norm_valid = false;
   // row-major copy
   int64_t* rowptr = nullptr;
   int32_t* colind = nullptr;
@@ -342,7 +352,14 @@ struct head_choice {
   bool fits = true;        // footprint within the budget given
 };
 constexpr double NO_BUDGET = 1e300;
-int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_blocks, head_choice* out);
+// rank > 0: the footprint also counts the head's workspace at that rank
+int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_blocks, int rank, head_choice* out);
+int64_t head_workspace_floats(int64_t n_rows, int64_t n_d, int r);
+// Sizes that the memory plan shares with the code that allocates (loader.hip).
+constexpr double PANEL_PARTIALS_BYTES = 3.0e9;  // the plain panels' partial sums stay within this
+int64_t coarse_panels_for(int64_t n_rows, int64_t n_cols, int r, bool sweeps);
+bool sweeps_for_rank(int r);
+int max_panels();
 // Dense blocks that the head's products at rank r read (1 or 2), see dense_head::rm.
 int head_blocks_for_rank(int r);
 int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense);

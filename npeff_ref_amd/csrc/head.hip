@@ -550,16 +550,26 @@ static int64_t head_slices_t(const dense_head& h, int r, int64_t n) {
   return head_slices_for((h.n_d_pad / 128) * ceil_div(r, 128), n);
 }
 
+// Floats of the workspace that the products of a head of n_d columns over n_rows rows use at rank r:
+// the gathered rows of H of the head, or W transposed (the split-operand product wants the
+// contraction index fast), plus the slice partials of the larger of the two products.
+int64_t head_workspace_floats(int64_t n_rows, int64_t n_d, int r) {
+  if (n_d <= 0) return 0;
+  dense_head h;
+  h.n_d = n_d;
+  h.n_d_pad = ceil_div(n_d, 128) * 128;
+  h.n_pad = ceil_div(n_rows, 128) * 128;
+  const int64_t gather = head_gather_floats(h, r);
+  const int64_t wn = head_slices_n(h, r) * h.n_pad * r;
+  const int64_t wt = head_slices_t(h, r, n_rows) * h.n_d_pad * r;
+  return gather + (wn > wt ? wn : wt);
+}
+
 int head_ensure_workspace(dnpeff_csr* A, int r) {
   dense_head& h = A->head;
   if (h.n_d == 0) return 0;
   DN_CHECK(r % 4 == 0, "a matrix with a dense head needs a rank that is a multiple of 4 (got %d)", r);
-  // gathered rows of H of the head, or W transposed (the split-operand product wants the
-  // contraction index fast)
-  const int64_t gather = head_gather_floats(h, r);
-  const int64_t wn = head_slices_n(h, r) * h.n_pad * r;
-  const int64_t wt = head_slices_t(h, r, A->n_rows) * h.n_d_pad * r;
-  const int64_t need = gather + (wn > wt ? wn : wt);
+  const int64_t need = head_workspace_floats(A->n_rows, h.n_d, r);
   if (!head_uses_split(r) && !h.rm) {  // the fp32 kernel of A^T W wants the block row by row
     if (dmalloc(&h.rm, h.n_pad * h.n_d_pad)) {
       // no room for the second copy: at ranks that the split-operand kernel handles the head's

@@ -60,12 +60,17 @@ int main(int argc, char** argv) {
   h5io::PefDims dims = h5io::pef_dims(flags.pef_path, flags.n_examples, flags.n_fisher_values);
   const long nnz_in = dims.n_rows * dims.n_values_per_row;
   // Row offsets are always 64-bit and column ids 32-bit inside the library; the reference's
-  // choice of index type (run_nmf_on_pefs.cu:236-244) still decides the log line and the type of
-  // reduce_kept_indices / full_dense_size in the output file (nmf_decomp_h5.h:58-75).
+  // choice of index type still decides the log lines and the type of reduce_kept_indices /
+  // full_dense_size in the output file (nmf_decomp_h5.h:58-75).  The reference chooses in two
+  // steps (run_nmf_on_pefs.cu:236-254): it reads with 64-bit indices when n_examples x
+  // n_fisher_values exceeds INT32_MAX, and then runs and saves with 32-bit ones when
+  // canReindexWithInt32() says so, which (matrices.h:219-224) is when the pruned matrix still holds
+  // more than INT32_MAX entries; only a matrix that pruning brought under INT32_MAX is run and
+  // saved with 64-bit indices.  The same file types come out here; --index_width overrides.
   if (flags.index_width != 0 && flags.index_width != 32 && flags.index_width != 64)
     fatal("Error: --index_width must be 32 or 64.");
-  const bool wide_indices = flags.index_width ? flags.index_width == 64 : nnz_in > (long)INT32_MAX;
-  if (wide_indices)
+  const bool read_wide = nnz_in > (long)INT32_MAX;
+  if (read_wide)
     std::cout << "Reading in PEFs using 64 bit indices.\n";
   else
     std::cout << "Using 32 bit indices.\n";
@@ -92,6 +97,10 @@ int main(int argc, char** argv) {
   ck(dnpeff_csr_shape(A, &n, &m, &nnz));
   std::cout << "n_cols after reduction: " << m << " [density=" << (double)nnz / (double)(n * m)
             << "]\n";
+
+  bool wide_indices = read_wide && !(nnz > (int64_t)INT32_MAX);
+  if (flags.index_width) wide_indices = flags.index_width == 64;
+  std::cout << (wide_indices ? "Running NMF using 64 bit indices.\n" : "Running NMF using 32 bit indices.\n");
 
   std::cout << "Initializing NMF.\n";
   dnpeff_nmf* nmf = nullptr;

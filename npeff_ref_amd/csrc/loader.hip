@@ -30,7 +30,12 @@ void set_error(const char* fmt, ...) {
 }
 void clear_error() { g_error[0] = 0; }
 
+static hipStream_t g_side_stream = nullptr;
+static bool g_on_side_stream = false;
+static hipEvent_t g_side_done = nullptr;  // recorded on the side stream; nullptr = nothing pending
+
 hipStream_t stream() {
+  if (g_on_side_stream) return g_side_stream;
   if (!g_stream) {
     if (hipStreamCreate(&g_stream) != hipSuccess) {
       fprintf(stderr, "dnpeff: hipStreamCreate failed (no usable GPU?)\n");
@@ -38,6 +43,35 @@ hipStream_t stream() {
     }
   }
   return g_stream;
+}
+
+// Work launched between side_stream_begin() and side_stream_end() goes to a second stream of the
+// same (default) priority: it starts once everything launched so far on the library stream has
+// finished, and runs beside what the library stream gets afterwards, until side_stream_join()
+// makes the library stream wait for it.
+int side_stream_begin() {
+  if (!g_side_stream) DN_HIP(hipStreamCreate(&g_side_stream));
+  static hipEvent_t fork = nullptr;
+  if (!fork) DN_HIP(hipEventCreateWithFlags(&fork, hipEventDisableTiming));
+  DN_HIP(hipEventRecord(fork, stream()));
+  DN_HIP(hipStreamWaitEvent(g_side_stream, fork, 0));
+  g_on_side_stream = true;
+  return 0;
+}
+int side_stream_end() {
+  static hipEvent_t done = nullptr;
+  if (!done) DN_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+  g_on_side_stream = false;
+  DN_HIP(hipEventRecord(done, g_side_stream));
+  g_side_done = done;
+  return 0;
+}
+int side_stream_join() {
+  if (!g_side_done) return 0;
+  hipEvent_t e = g_side_done;
+  g_side_done = nullptr;
+  DN_HIP(hipStreamWaitEvent(stream(), e, 0));
+  return 0;
 }
 
 int n_cus() {
@@ -64,6 +98,7 @@ static const tuning_entry g_tuning_table[] = {
     {"n_lists", &tuning_t::n_lists},             {"t_lists", &tuning_t::t_lists},
     {"nl_piece_cols", &tuning_t::nl_piece_cols}, {"nl_lag", &tuning_t::nl_lag},
     {"nl_spin", &tuning_t::nl_spin},             {"nl_wgs", &tuning_t::nl_wgs},
+    {"gram_beside", &tuning_t::gram_beside},
 };
 
 static tuning_t tuning_from_env() {
@@ -226,17 +261,19 @@ __global__ void __launch_bounds__(256)
     table[i] = og_to_new[i] >= 0 ? -1 : (int32_t)i;
 }
 
-// Entries of the head's columns into the dense block; a workgroup per row.  (A matrix whose rows
-// hold a column twice is refused by the products, so every element receives one addition.)
+// Entries of the head's columns into the dense block; a workgroup per row.  Every element must
+// receive one addition: an addition that finds something other than zero in its element means
+// that the row holds the column twice (*repeats counts them; a repeat whose earlier values were
+// all exactly zero goes unnoticed and changes nothing: 0 + x has one value whatever the order).
 __global__ void __launch_bounds__(256)
     k_head_fill(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
                 const float* __restrict__ vals, int64_t n_rows, const int32_t* __restrict__ slot_of,
-                float* __restrict__ cm, int64_t n_pad) {
+                float* __restrict__ cm, int64_t n_pad, int* __restrict__ repeats) {
   for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
     const int64_t e1 = rowptr[row + 1];
     for (int64_t e = rowptr[row] + threadIdx.x; e < e1; e += 256) {
       const int32_t k = slot_of[colind[e]];
-      if (k >= 0) atomicAdd(&cm[(int64_t)k * n_pad + row], vals[e]);
+      if (k >= 0 && atomicAdd(&cm[(int64_t)k * n_pad + row], vals[e]) != 0.0f) atomicAdd(repeats, 1);
     }
   }
 }
@@ -697,25 +734,35 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
 // The `panels` switch overrides the number (0 = none).  Swept pieces hold `sweep_bytes` of the
 // factor each (default 3 MB of the 4 MB L2 of an XCD; 0 = no sweeps) and are made where a row
 // holds `sweep_min` entries per piece on average (default 4, more when there are few rows).
-static panel_plan panel_policy(const dnpeff_csr* S, int r) {
+// Coarse panels for a sparse part of n_rows x n_cols at rank r (0 = none); `sweeps`: the rank and
+// the machine have swept pieces.
+int64_t coarse_panels_for(int64_t n_rows, int64_t n_cols, int r, bool sweeps) {
   const tuning_t& tn = tuning();
   int64_t P = 0;
-  const double bytes = 4.0 * (double)S->n_cols * r;
-  const bool sweeps = spmm_n_sweep_supported(r) && tn.sweep_bytes > 0.0 && xcd_round_robin();
-  if (bytes >= 512e6 && S->n_rows >= 64) {
+  const double bytes = 4.0 * (double)n_cols * r;
+  if (bytes >= 512e6 && n_rows >= 64) {
     // with swept pieces for the panels in between, half as many coarse panels do as well for the
     // gathers and halve the sum over the panels (configs[1]: 19.8 -> 19.4 ms for both)
     P = (int64_t)ceil(bytes / (sweeps ? 96e6 : 48e6));
     if (P < 8) P = 8;
     if (P > (sweeps ? 256 : 512)) P = sweeps ? 256 : 512;
-    const int64_t by_partials = (int64_t)(3.0e9 / (4.0 * (double)S->n_rows * r));
+    const int64_t by_partials = (int64_t)(PANEL_PARTIALS_BYTES / (4.0 * (double)n_rows * r));
     if (P > by_partials) P = by_partials < 8 ? 8 : by_partials;
   }
   if (tn.panels >= 0.0) P = (int64_t)tn.panels;
   if (P > 512) P = 512;
-  const int64_t row_groups = ceil_div(S->n_rows, 4);
+  const int64_t row_groups = ceil_div(n_rows, 4);
   while (P > 1 && P * row_groups >= ((int64_t)1 << 24)) P /= 2;
-  if (P < 2 || S->nnz == 0) P = 0;
+  return P < 2 ? 0 : P;
+}
+bool sweeps_for_rank(int r) { return spmm_n_sweep_supported(r) && tuning().sweep_bytes > 0.0 && xcd_round_robin(); }
+int max_panels() { return MAX_PANELS; }
+
+static panel_plan panel_policy(const dnpeff_csr* S, int r) {
+  const tuning_t& tn = tuning();
+  const bool sweeps = sweeps_for_rank(r);
+  int64_t P = coarse_panels_for(S->n_rows, S->n_cols, r, sweeps);
+  if (S->nnz == 0) P = 0;
   panel_plan plan;
   plan.coarse = (int)P;
   if (P > 0 && sweeps) {
@@ -1028,6 +1075,7 @@ DN_API int dnpeff_csr_normalize_rows(dnpeff_csr* A, const float* norms_host, flo
   DN_HIP(hipStreamSynchronize(stream()));
   dfree(norms);
   drop_derived(A);
+  A->sq_norm_valid = false;
   return 0;
 }
 
@@ -1036,6 +1084,7 @@ DN_API int dnpeff_csr_compact_columns(dnpeff_csr* A, int min_count) {
   DN_CHECK(A && has_row_major(A), "matrix is NULL or its row-major arrays were released");
   hipStream_t st = stream();
   drop_derived(A);
+  A->sq_norm_valid = false;
   const int64_t m_full = A->n_cols;
   dbuf<int> count;
   dbuf<int32_t> pos, og_to_new, new_to_og;
@@ -1072,6 +1121,7 @@ DN_API int dnpeff_csr_retain_columns(dnpeff_csr* A, const int32_t* kept, int64_t
              (long long)i, kept[i], (long long)A->n_cols);
   hipStream_t st = stream();
   drop_derived(A);
+  A->sq_norm_valid = false;
   int32_t *table = nullptr, *kept_dev = nullptr;
   DN_TRY(dmalloc(&table, A->n_cols));
   DN_TRY(dmalloc(&kept_dev, n_kept));
@@ -1131,8 +1181,13 @@ DN_API int dnpeff_csr_kept_indices(const dnpeff_csr* A, int32_t* new_to_og) {
 DN_API int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out) {
   clear_error();
   DN_CHECK(A && out, "NULL argument");
-  const float* v = A->vals ? A->vals : A->tvals;
-  DN_CHECK(v != nullptr || A->nnz == 0, "both copies of the matrix were released");
+  if (A->sq_norm_valid) {
+    *out = A->sq_norm;
+    return 0;
+  }
+  // (with a dense head the whole matrix's values only exist in the row-major copy)
+  const float* v = A->vals ? A->vals : (A->tail ? nullptr : A->tvals);
+  DN_CHECK(v != nullptr || A->nnz == 0, "the row-major copy of the matrix was released before its norm was taken");
   const int blocks = 1024;
   double* partials = nullptr;
   DN_TRY(dmalloc(&partials, blocks));
@@ -1144,6 +1199,9 @@ DN_API int dnpeff_csr_sq_norm(const dnpeff_csr* A, double* out) {
   double s = 0.0;
   for (int i = 0; i < blocks; i++) s += h[i];
   *out = s;
+  dnpeff_csr* M = const_cast<dnpeff_csr*>(A);
+  M->sq_norm = s;
+  M->sq_norm_valid = true;
   return 0;
 }
 
@@ -1165,7 +1223,7 @@ namespace dn {
 // the remaining entries (16 bytes each).  The choice is the first admissible candidate
 // whose footprint is within `budget` bytes (NO_BUDGET: the first admissible one), else the
 // admissible candidate with the smallest footprint (fits = false).
-int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_blocks, head_choice* out) {
+int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_blocks, int rank, head_choice* out) {
   *out = head_choice();
   out->footprint = 16.0 * (double)A->nnz;
   out->fits = out->footprint <= budget;
@@ -1207,7 +1265,8 @@ int choose_dense_head(dnpeff_csr* A, double min_fill, double budget, int n_block
     head_choice c;
     c.thr = thr;
     c.n_d = n_d;
-    c.footprint = blocks + 16.0 * (double)(A->nnz - (int64_t)z_head);
+    c.footprint = blocks + 16.0 * (double)(A->nnz - (int64_t)z_head) +
+                  (rank > 0 ? 4.0 * (double)head_workspace_floats(n, n_d, rank) : 0.0);
     c.fits = c.footprint <= budget;
     if (c.fits) {
       best = c;
@@ -1255,9 +1314,20 @@ int split_dense_head_at(dnpeff_csr* A, int64_t thr, int64_t* n_dense) {
   dbuf<float> cm;
   DN_TRY(cm.alloc(n_d_pad * n_pad));
   DN_HIP(hipMemsetAsync(cm, 0, sizeof(float) * (size_t)(n_d_pad * n_pad), st));
-  hipLaunchKernelGGL(k_head_fill, dim3(grid_for(n * 256)), dim3(256), 0, st, A->rowptr, A->colind,
-                     A->vals, n, slot_of.p, cm.p, n_pad);
-  DN_LAUNCH_CHECK();
+  {
+    dbuf<int> repeats;
+    DN_TRY(repeats.alloc(1));
+    DN_HIP(hipMemsetAsync(repeats, 0, sizeof(int), st));
+    hipLaunchKernelGGL(k_head_fill, dim3(grid_for(n * 256)), dim3(256), 0, st, A->rowptr, A->colind,
+                       A->vals, n, slot_of.p, cm.p, n_pad, repeats.p);
+    DN_LAUNCH_CHECK();
+    int n_rep = 0;
+    DN_HIP(hipMemcpy(&n_rep, repeats.p, sizeof(int), hipMemcpyDeviceToHost));
+    DN_CHECK(n_rep == 0,
+             "%d entries of the dense head's columns repeat a (row, column) pair: duplicate entries are "
+             "not supported by the products",
+             n_rep);
+  }
   // the remaining entries: the row-major arrays without the head's columns, written straight
   // into the tail's own arrays (positions from a scan over the entries)
   dnpeff_csr* T = new dnpeff_csr();
@@ -1307,7 +1377,7 @@ DN_API int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* 
     return 0;
   }
   head_choice c;
-  DN_TRY(choose_dense_head(A, min_fill, NO_BUDGET, 2, &c));
+  DN_TRY(choose_dense_head(A, min_fill, NO_BUDGET, 2, 0, &c));
   return split_dense_head_at(A, c.thr, n_dense);
 }
 

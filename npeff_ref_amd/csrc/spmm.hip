@@ -1139,7 +1139,11 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
       });
       DN_LAUNCH_CHECK();
     }
-    if (A->n_swept > 0) DN_TRY(launch_spmm_n_sweep(A, r, H_mr, aligned, slots));
+    // (the sweep kernel wants the CUs to itself: all its workgroups must be resident)
+    if (A->n_swept > 0) {
+      DN_TRY(side_stream_join());
+      DN_TRY(launch_spmm_n_sweep(A, r, H_mr, aligned, slots));
+    }
     return 0;
   }
   DN_CHECK(A->rowptr && A->chunk_base && partials, "matrix has no row-major copy / work list");

@@ -149,3 +149,40 @@ def test_bench_work_model_and_sample_sizes():
     assert held and got == held[0] and got > 8 * z and src == "profiles/nmf_c3_hbm_traffic.md"
     assert bench.traffic_from_profile("c3", "no_such_class") == (None, None)
     assert bench.traffic_from_profile("c0", "spmm_n") == (None, None)
+
+
+def test_memory_plan_arithmetic_for_the_benchmark_shapes():
+    """dnpeff_plan_estimate needs no GPU: the byte table of the memory plan for the shapes of
+    BASELINE configs[1], [3] and [4] as generated (kept columns, entries of the sparse part and head
+    columns as the full-size runs report them) follows the sizing rules, fits the 309.2 GB the
+    device reports, and prices a larger head higher."""
+    total = 309_220_868_096
+    n, m, r = 20_000, 211_311_151, 256
+    c3 = d.plan_estimate(n, m, 2_355_000_000, 437_520, r, tiled=True, total_bytes=total)
+    full = d.plan_estimate(n, m, 2_355_000_000, 437_520, r, tiled=False, total_bytes=total)
+    tile = (768 * 2**20 // (4 * r)) // 128 * 128  # h_tile_mb = 768 MiB of the factor, a multiple of 128 columns
+    assert tile == 786_432
+    # full-size: H and A^T W as two [m, r] arrays; tiled: [m + tile, r] and [tile, r]
+    assert full["factors"] - c3["factors"] == 4.0 * r * (m - 2 * tile)
+    assert c3["factors"] > 4.0 * r * (m + 2 * tile) + 3 * 4.0 * n * r
+    # plain panels capped so that their partial sums stay within 3 GB, plus one set per XCD
+    panels = int(3.0e9 // (4 * n * r))
+    assert panels == 146 and c3["partials"] == 4.0 * r * n * (panels + 8)
+    assert c3["segments"] == 8.0 * n * (3072 + 1)
+    assert 8.0 * (m + 1) < c3["offsets"] < 8.5 * (m + 1)
+    assert c3["reserve"] == total / 64
+    assert c3["sparse_copies"] == 16.0 * 2_355_000_000
+    assert c3["head_blocks"] == 4.0 * 20_096 * 437_632  # one block, rows and columns padded to 128
+    assert 0 < c3["head_workspace"] < 0.1 * c3["head_blocks"]
+    assert sum(c3.values()) < total < sum(full.values())  # only the tiled update fits
+    bigger = d.plan_estimate(n, m, 2_000_000_000, 600_000, r, tiled=True, total_bytes=total)
+    assert bigger["head_blocks"] > c3["head_blocks"] and bigger["head_workspace"] >= c3["head_workspace"]
+    assert sum(bigger.values()) > total  # the head at fill 1/16 does not fit beside H: the threshold rises
+    c1 = d.plan_estimate(10_000, 65_941_155, 382_000_000, 120_802, 128, tiled=False, total_bytes=total)
+    assert sum(c1.values()) < 0.3 * total and c1["head_blocks"] == 2 * 4.0 * 10_112 * 120_832 / 2
+    c4 = d.plan_estimate(40_000, 107_300_000, 2_000_000_000, 100_000, 512, tiled=True, total_bytes=total)
+    assert sum(c4.values()) < total
+    # a small device: the reserve never goes below 1 GiB
+    assert d.plan_estimate(512, 900_000, 2_097_152, 0, 16, False, total_bytes=8 * 2**30)["reserve"] == 2.0**30
+    with pytest.raises(d.DnpeffError):
+        d.plan_estimate(10, 5, 1, 6, 16, False)  # more head columns than columns

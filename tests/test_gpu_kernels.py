@@ -285,6 +285,10 @@ def test_duplicate_entries_are_refused_by_the_products():
     H = d.DeviceArray.from_numpy(rng.random((3000, 64)).astype(np.float32))
     with pytest.raises(d.DnpeffError, match="duplicate"):
         d.op_spmm_n(A, 64, H, d.DeviceArray((200, 64)))
+    # the repeated pairs sit in columns that most rows hold: moving those to the dense head (which
+    # would otherwise add them up, in an order of the hardware's choosing) finds them too
+    with pytest.raises(d.DnpeffError, match="duplicate"):
+        A.split_dense_head(0.5)
     A.close()
 
 

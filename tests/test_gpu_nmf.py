@@ -127,6 +127,52 @@ def test_loss_evaluations_do_not_change_the_run(rank):
     assert outs[0][2] == outs[1][2] == outs[1][3][-1] == outs[1][3][-2]
 
 
+@pytest.mark.parametrize("rank,n", [(256, 1500), (64, 300)])
+def test_gram_beside_the_sparse_product_gives_the_same_bits(rank, n, tune):
+    """The gram_beside switch only moves H^T H of the W update to a second stream, beside A H^T: the
+    same kernels on the same operands, so six iterations end on the same bits (rank 256 with a
+    dense head, panels and swept pieces forced on; rank 64 without)."""
+    outs = []
+    for beside in (0, 1):
+        tune("gram_beside", beside)
+        tune("panels", 8)
+        tune("sweep_bytes", 300 * 4 * min(rank, 256))
+        tune("sweep_min", 0)
+        A, norms = d.Csr.synth(n, 200000, k_fixed=1500, zipf_s=1.3, seed=21)
+        A.normalize_rows(norms)
+        A.compact_columns(1)
+        nmf = d.MuNmf(A, d.MuNmfParams(rank=rank, max_iters=6, log_every=3))
+        nmf.initialize()
+        hist = nmf.run(log=lambda s: None)
+        outs.append((nmf.loadWToHostSync(), nmf.loadHToHostSync(), [h[1] for h in hist]))
+        nmf.close()
+        A.close()
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    assert outs[0][2] == outs[1][2]
+
+
+@pytest.mark.parametrize("fill", [1.0 / 16.0, 0.0])
+def test_second_context_on_a_consumed_matrix(fill, tune):
+    """A matrix whose arrays a consuming create has released still serves a later context of the
+    same rank (with a dense head: only head and tail are left; without: only the transposed and
+    regrouped copies): same ||A||^2, same factors, same loss, bit for bit."""
+    tune("dense_fill", fill)
+    A, norms = d.Csr.synth(1500, 200000, k_fixed=1500, zipf_s=1.3, seed=33)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    outs = []
+    for _ in range(2):
+        nmf = d.MuNmf(A, d.MuNmfParams(rank=128, max_iters=3, log_every=0), consume_matrix=True)
+        assert (A.head_info()[0] > 0) == (fill > 0)
+        nmf.initialize()
+        nmf.step(3)
+        outs.append((nmf.loss_terms(), nmf.loadWToHostSync(), nmf.loadHToHostSync()))
+        nmf.close()
+    assert outs[0][0] == outs[1][0]
+    assert np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][2], outs[1][2])
+    A.close()
+
+
 def test_more_rows_than_columns_is_refused():
     A = d.Csr.from_host([0, 1, 2, 3], [0, 1, 0], [1.0, 1.0, 1.0], 2)
     with pytest.raises(d.DnpeffError, match="more rows than columns"):

@@ -116,17 +116,20 @@ def test_run_nmf_on_pefs_end_to_end(tmp_path):
 
 @pytest.mark.gpu
 def test_run_nmf_on_pefs_wide_index_schema(tmp_path):
-    """The reference instantiates its writer with IndT = int64 when n_examples x n_fisher_values
-    exceeds INT32_MAX (nmf_decomp_h5.h:58-75): reduce_kept_indices and full_dense_size are then
-    int64.  --index_width=64 forces that branch on a small file; the values are the same, and
-    the fit path reads such a file."""
+    """The reference's writer with IndT = int64 (nmf_decomp_h5.h:58-75) stores reduce_kept_indices and
+    full_dense_size as int64; it is reached when the PEF file was read with 64-bit indices and
+    the pruned matrix holds no more than INT32_MAX entries (run_nmf_on_pefs.cu:236-247 with
+    matrices.h:219-224).  --index_width=64 forces that branch on a small file; the values are the
+    same, and the fit path reads such a file."""
     n, m_full, k, r = 24, 9000, 300, 8
     pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=5)
     out32, out64 = str(tmp_path / "d32.h5"), str(tmp_path / "d64.h5")
     common = [f"--per_example_fishers={pef}", f"--nmf_n_components={r}", "--nmf_max_iter=3"]
-    run("run_nmf_on_pefs", f"--output_path={out32}", *common, check=True)
+    p = run("run_nmf_on_pefs", f"--output_path={out32}", *common, check=True)
+    assert "Using 32 bit indices." in p.stdout.splitlines()
+    assert "Running NMF using 32 bit indices." in p.stdout.splitlines()
     p = run("run_nmf_on_pefs", f"--output_path={out64}", "--index_width=64", *common, check=True)
-    assert "Reading in PEFs using 64 bit indices." in p.stdout.splitlines()
+    assert "Running NMF using 64 bit indices." in p.stdout.splitlines()
     k32, k64 = h5lite.read(out32, "data/reduce_kept_indices"), h5lite.read(out64, "data/reduce_kept_indices")
     assert k32.dtype == np.int32 and k64.dtype == np.int64 and np.array_equal(k32, k64)
     f32, s32 = h5lite.attr(out32, "data/reduce_kept_indices", "full_dense_size")

@@ -64,3 +64,14 @@ def test_static_gram_refuses_what_does_not_fit():
         d.binding._check(d.lib.dnpeff_op_gram_static(64, 256, X.ptr, G.ptr))
     with pytest.raises(d.DnpeffError):
         d.binding._check(d.lib.dnpeff_op_gram_static(0, 128, X.ptr, G.ptr))
+
+
+def test_static_gram_takes_any_row_count_at_small_ranks():
+    """At ranks up to 32 the partial sums are one 32 x 32 block per workgroup, at most 512 of them:
+    row counts far past the limit of the larger ranks fit the scratch array."""
+    rng = np.random.default_rng(3)
+    X = rng.random((150_000, 16), dtype=np.float32)
+    ref, got = _both(X, 150_000, 16)
+    assert np.array_equal(ref, got)
+    want = X.astype(np.float64).T @ X.astype(np.float64)
+    assert np.max(np.abs(got - want) / np.abs(want)) < 2e-6
