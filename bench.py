@@ -239,45 +239,54 @@ def run_scipy_baseline(sample, n, m, z, r, eps, max_entries=3.0e7):
 # dense-factor NMF (run_nmf_on_pefs)
 # ------------------------------------------------------------------------------------------
 def compare_decompositions(d, cfg, seed, r):
-    """A H^T on the first rows of the ragged matrix under three work decompositions of the sparse
-    part: one wavefront per row, 2048-entry row chunks (the merge-path split for rows this long),
-    and the planned one (column panels + swept pieces + dense head)."""
+    """A H^T on the first rows of the ragged matrix under four work decompositions of the sparse
+    part: one wavefront per row, 2048-entry row chunks, the merge path (equal shares of entries +
+    rows, cut wherever the row boundaries fall) and the planned one (column panels + swept pieces
+    + dense head).  Twice: with the row lengths of the configuration (1,024 .. 524,288, where a
+    chunk split is the merge path up to the last, shorter chunk of each row) and with lengths from
+    16 up, where thousands of short rows separate the two."""
     rows = cfg.get("compare_rows")
     if not rows:
         return None
-    A, norms = d.Csr.synth(rows, cfg["m_full"], k_fixed=cfg["k"], k_min=cfg["kmin"], k_max=cfg["kmax"],
-                           zipf_s=cfg["s"], seed=seed)
-    A.normalize_rows(norms)
-    A.compact_columns(1)
-    n, m, z = A.n_rows, A.n_cols, A.nnz
-    lens = np.diff(A.download()[0])
-    hist, edges = np.histogram(np.log2(lens), bins=np.arange(10, 20.01, 1.0))
-    H = d.DeviceArray((m, r))
-    d.op_init_uniform(0, m, r, seed, H)
-    N = d.DeviceArray((n, r))
-    out = {"rows": n, "columns": m, "entries": z, "rank": r,
-           "row_length_histogram_log2": {f"2^{int(a)}..2^{int(b)}": int(c) for a, b, c in zip(edges[:-1], edges[1:], hist)},
-           "row_length_min_max": [int(lens.min()), int(lens.max())]}
-    ref = None
-    for variant, name in ((1, "wave_per_row"), (2, "row_chunks_2048"), (0, "planned_panels_sweeps_head")):
-        for _ in range(2):
-            d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, H.ptr, N.ptr, variant))
-        d.sync()
-        t0 = time.perf_counter()
-        reps = 3
-        for _ in range(reps):
-            d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, H.ptr, N.ptr, variant))
-        d.sync()
-        ms = (time.perf_counter() - t0) * 1e3 / reps
-        got = N.numpy()
-        if ref is None:
-            ref = got.astype(np.float64)
-        err = float(np.max(np.abs(got - ref)) / np.max(np.abs(ref)))
-        out[name] = {"ms": ms, "max_rel_diff_vs_wave_per_row": err}
-        log(f"  A H^T on {n} ragged rows ({z} entries), {name}: {ms:.2f} ms (diff {err:.1e})")
-    dense_cols, z_sparse = A.head_info()
-    out["dense_head_columns"], out["entries_sparse_part"] = dense_cols, z_sparse
-    H.free(); N.free(); A.close()
+    out = {}
+    for label, kmin in (("as_configured", cfg["kmin"]), ("short_rows_too", 16)):
+        A, norms = d.Csr.synth(rows, cfg["m_full"], k_fixed=cfg["k"], k_min=kmin, k_max=cfg["kmax"],
+                               zipf_s=cfg["s"], seed=seed)
+        A.normalize_rows(norms)
+        A.compact_columns(1)
+        n, m, z = A.n_rows, A.n_cols, A.nnz
+        lens = np.diff(A.download()[0])
+        hist, edges = np.histogram(np.log2(lens), bins=np.arange(4, 20.01, 2.0))
+        H = d.DeviceArray((m, r))
+        d.op_init_uniform(0, m, r, seed, H)
+        N = d.DeviceArray((n, r))
+        res = {"rows": n, "columns": m, "entries": z, "rank": r,
+               "row_length_histogram_log2": {f"2^{int(a)}..2^{int(b)}": int(c)
+                                             for a, b, c in zip(edges[:-1], edges[1:], hist)},
+               "row_length_min_max": [int(lens.min()), int(lens.max())]}
+        ref = None
+        for variant, name in ((1, "wave_per_row"), (2, "row_chunks_2048"), (3, "merge_path_4096"),
+                              (0, "planned_panels_sweeps_head")):
+            for _ in range(2):
+                d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, H.ptr, N.ptr, variant))
+            d.sync()
+            t0 = time.perf_counter()
+            reps = 3
+            for _ in range(reps):
+                d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, H.ptr, N.ptr, variant))
+            d.sync()
+            ms = (time.perf_counter() - t0) * 1e3 / reps
+            got = N.numpy()
+            if ref is None:
+                ref = got.astype(np.float64)
+            err = float(np.max(np.abs(got - ref)) / np.max(np.abs(ref)))
+            res[name] = {"ms": ms, "max_rel_diff_vs_wave_per_row": err}
+            log(f"  A H^T on {n} ragged rows of {lens.min()}..{lens.max()} entries ({z} in all), {name}: "
+                f"{ms:.2f} ms (diff {err:.1e})")
+        dense_cols, z_sparse = A.head_info()
+        res["dense_head_columns"], res["entries_sparse_part"] = dense_cols, z_sparse
+        H.free(); N.free(); A.close()
+        out[label] = res
     return out
 
 

@@ -377,8 +377,11 @@ int dnpeff_op_spmm_n(dnpeff_csr* A, int r, const float* H_mr, float* N_nr);
 /* The same product with the work decomposition of the sparse part chosen by the caller, for
  * comparisons on ragged rows: 0 = as planned (column panels and swept pieces where the factor
  * is large, else row chunks), 1 = one wavefront per row, 2 = chunks of 2048 entries of a row with
- * a second pass over the chunk sums (with rows of 1024 entries and more this is the merge-path
- * split up to the last, shorter chunk of each row).  1 and 2 need the row-major arrays. */
+ * a second pass over the chunk sums, 3 = merge path: every wavefront takes 4096 consecutive steps
+ * of the path that consumes each row's entries and then its end marker, wherever the row
+ * boundaries fall (the nnz-balanced split of cc/cuda_d_npeff/src/cuda/ops/sp_slicing.h:314-403
+ * taken down to wavefronts), with a pass that adds the sums of the rows cut between shares.
+ * 1, 2 and 3 need the row-major arrays. */
 int dnpeff_op_spmm_n_variant(dnpeff_csr* A, int r, const float* H_mr, float* N_nr, int variant);
 
 /* T[m, r] = A^T W with W [n, r]; needs dnpeff_csr_build_transpose.

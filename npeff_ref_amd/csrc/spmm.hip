@@ -245,6 +245,69 @@ __global__ void __launch_bounds__(256)
 }
 
 // ---------------------------------------------------------------------------
+// Merge-path decomposition, for the comparison of work decompositions on ragged rows: the path
+// that consumes, row by row, a row's entries and then its end marker has nnz + n_rows steps; every
+// wave takes MERGE_SHARE consecutive steps of it, wherever the row boundaries fall (a long row is
+// cut over many waves, many short rows share one).  Diagonal d of the path lies at (rows closed,
+// entries consumed) = (i, d - i) with i = the number of rows whose end marker, at step
+// rowptr[i + 1] + i, comes before d.  A row that starts and ends inside a share is stored directly;
+// the share's sums for the row that was open when it began / that stays open when it ends go to
+// carry[share][0] / [1] and k_merge_fixup adds a row's carries in share order.
+// ---------------------------------------------------------------------------
+constexpr int64_t MERGE_SHARE = 4096;
+
+__device__ inline int64_t merge_rows_closed(const int64_t* __restrict__ rowptr, int64_t n_rows, int64_t d) {
+  int64_t lo = 0, hi = n_rows;  // number of i in [0, n_rows) with rowptr[i + 1] + i < d
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (rowptr[mid + 1] + mid < d) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+template <class GT>
+__global__ void __launch_bounds__(256)
+    k_spmm_n_merge(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
+                   const float* __restrict__ vals, int64_t n_rows, int64_t n_shares, int r,
+                   const float* __restrict__ H, float* __restrict__ N, float* __restrict__ carry) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int64_t share = (int64_t)blockIdx.x * 4 + wave;
+  if (share >= n_shares) return;
+  const int64_t total = rowptr[n_rows] + n_rows;
+  const int64_t d0 = share * MERGE_SHARE, d1 = d0 + MERGE_SHARE < total ? d0 + MERGE_SHARE : total;
+  const int64_t i0 = merge_rows_closed(rowptr, n_rows, d0), i1 = merge_rows_closed(rowptr, n_rows, d1);
+  const int64_t e0 = d0 - i0, e1 = d1 - i1;
+  for (int64_t i = i0; i <= i1 && i < n_rows; i++) {
+    const int64_t r0 = rowptr[i], r1 = rowptr[i + 1];
+    const int64_t a = r0 > e0 ? r0 : e0, b = r1 < e1 ? r1 : e1;
+    const bool opened_before = r0 < e0, closes_here = i < i1;
+    if (i == i1 && !opened_before && b <= a && r0 >= e1) break;  // the next share's row: nothing of it here
+    GT g;
+    g.init(lane, r);
+    g.run(colind, vals, a, b > a ? b : a, H, r);
+    if (!opened_before && closes_here) g.store(N + i * r);
+    else g.store(carry + (share * 2 + (opened_before ? 0 : 1)) * r);
+  }
+}
+
+// N[row, :] of the rows that span several shares: the tail carry of the share where the row
+// starts, then the head carries of the following shares up to the one with its end marker.
+__global__ void __launch_bounds__(256)
+    k_merge_fixup(const int64_t* __restrict__ rowptr, int64_t n_rows, int r, const float* __restrict__ carry,
+                  float* __restrict__ N) {
+  for (int64_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
+    const int64_t sa = (rowptr[i] + i) / MERGE_SHARE, sb = (rowptr[i + 1] + i) / MERGE_SHARE;
+    if (sa == sb) continue;
+    // (a row whose first step is the first step of share sa was not open before it)
+    for (int c = threadIdx.x; c < r; c += 256) {
+      float s = carry[(sa * 2 + 1) * r + c];
+      for (int64_t sh = sa + 1; sh <= sb; sh++) s += carry[(sh * 2) * r + c];
+      N[i * r + c] = s;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Column panels.  When H is far larger than the caches, every gathered row of H comes from
 // HBM unless the workgroups running at one time gather from the same part of H.  The entries of
 // each row are therefore regrouped by column panel (same panels for all rows, equal numbers of
@@ -1349,7 +1412,8 @@ DN_API int dnpeff_op_spmm_n_variant(dnpeff_csr* A_full, int r, const float* H_mr
   DN_CHECK(A_full && H_mr && N_nr, "NULL argument");
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
   if (variant == 0) return dnpeff_op_spmm_n(A_full, r, H_mr, N_nr);
-  DN_CHECK(variant == 1 || variant == 2, "variant must be 0 (planned), 1 (a wave per row) or 2 (row chunks)");
+  DN_CHECK(variant >= 1 && variant <= 3,
+           "variant must be 0 (planned), 1 (a wave per row), 2 (row chunks) or 3 (merge path)");
   DN_TRY(csr_ensure_products(A_full, r));
   dnpeff_csr* A = sparse_part(A_full);
   DN_CHECK(has_row_major(A), "the row-major arrays of the sparse part were released");
@@ -1365,6 +1429,25 @@ DN_API int dnpeff_op_spmm_n_variant(dnpeff_csr* A_full, int r, const float* H_mr
         return 0;
       });
       DN_LAUNCH_CHECK();
+    }
+  } else if (variant == 3) {
+    const int64_t n_shares = ceil_div(A->nnz + A->n_rows, MERGE_SHARE);
+    if (n_shares > 0) {
+      dbuf<float> carry;
+      DN_TRY(carry.alloc(n_shares * 2 * (int64_t)r));
+      DN_CHECK(ceil_div(n_shares, 4) < ((int64_t)1 << 24), "too many shares for one launch");
+      dim3 grid((unsigned)ceil_div(n_shares, 4)), block(256);
+      dispatch_gather(r, aligned, [&](auto tag) {
+        using GT = typename decltype(tag)::type;
+        hipLaunchKernelGGL((k_spmm_n_merge<GT>), grid, block, 0, stream(), A->rowptr, A->colind, A->vals,
+                           A->n_rows, n_shares, r, H_mr, N_nr, carry.p);
+        return 0;
+      });
+      int64_t wgs = A->n_rows < 65536 ? A->n_rows : 65536;
+      hipLaunchKernelGGL(k_merge_fixup, dim3((unsigned)wgs), dim3(256), 0, stream(), A->rowptr, A->n_rows, r,
+                         carry.p, N_nr);
+      DN_LAUNCH_CHECK();
+      DN_HIP(hipStreamSynchronize(stream()));  // (the carries are freed on return)
     }
   } else {
     DN_TRY(csr_ensure_chunks(A));

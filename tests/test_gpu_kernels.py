@@ -491,18 +491,29 @@ def test_row_and_column_inspection_and_gathered_rows():
 
 @pytest.mark.parametrize("r", [64, 100, 512])
 def test_spmm_n_decompositions_agree(r, tune):
-    """One wave per row, 2048-entry row chunks and the planned decomposition (forced panels and
-    swept pieces) of A H^T on ragged rows: the same sums up to fp32 order, each against fp64."""
+    """One wave per row, 2048-entry row chunks, the merge path (equal shares of entries + rows,
+    cut wherever the row boundaries fall) and the planned decomposition (forced panels and swept
+    pieces) of A H^T on ragged rows, some of them empty: the same sums up to fp32 order, each
+    against fp64."""
     tune("panels", 8)
     tune("sweep_bytes", 300 * 4 * min(r, 256))
     tune("sweep_min", 0)
     rowptr, colind, vals, norms = d.synth_pef_host(300, 40000, k_min=8, k_max=6000, seed=r)
+    # rows 5, 6 and the last one emptied: end markers only on the merge path
+    keep = np.ones(len(colind), dtype=bool)
+    lens = np.diff(rowptr)
+    for i in (5, 6, 299):
+        keep[rowptr[i]:rowptr[i + 1]] = False
+        lens[i] = 0
+    colind, vals = colind[keep], vals[keep]
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
     A = d.Csr.from_host(rowptr, colind, vals, 40000)
     rng = np.random.default_rng(r)
     H = rng.random((40000, r)).astype(np.float32)
     dH, dN = d.DeviceArray.from_numpy(H), d.DeviceArray((300, r))
     N64 = orc.spmm_n_f64(rowptr, colind, vals, H)
-    for variant in (1, 2, 0):
+    for variant in (1, 2, 3, 0):
+        dN = d.DeviceArray.from_numpy(np.full((300, r), np.nan, dtype=np.float32))  # every element must be written
         d.binding._check(d.lib.dnpeff_op_spmm_n_variant(A._h, r, dH.ptr, dN.ptr, variant))
         d.sync()
         N = dN.numpy()
