@@ -70,6 +70,27 @@ def cpu_model():
     return platform.processor() or "unknown"
 
 
+def physical_cores():
+    """Distinct (package, core) pairs among the CPUs this process may run on; None where /proc does
+    not tell."""
+    try:
+        allowed = os.sched_getaffinity(0)
+        seen, cur = set(), {}
+        for line in open("/proc/cpuinfo"):
+            if ":" in line:
+                k, v = (x.strip() for x in line.split(":", 1))
+                cur[k] = v
+            elif cur:
+                if int(cur.get("processor", -1)) in allowed:
+                    seen.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+                cur = {}
+        if cur and int(cur.get("processor", -1)) in allowed:
+            seen.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+        return len(seen) or None
+    except Exception:
+        return None
+
+
 def algorithmic(cls, n, m, z, r, fused_gram=False, split_bf16=False):
     """Compulsory work of one product / update over the whole matrix, every operand touched once:
     (bytes, fp32 flops, split).  flops = 0 for the kernels without a matrix product.  With
@@ -133,9 +154,12 @@ def traffic_from_profile(config, cls):
 # ------------------------------------------------------------------------------------------
 # CPU baseline: the fp32 OpenMP port of the reference loop on the host cores, on a bounded sample
 # ------------------------------------------------------------------------------------------
-def cpu_sample_rows(cfg):
+def cpu_sample_rows(cfg, rows=0):
     """Rows of the sample: all of them while n k r stays within ~1e11 multiply-adds per product
-    (configs[1] in full), else the first rows of the matrix up to ~3.5e10."""
+    (configs[1] in full), else the first rows of the matrix up to ~3.5e10 (about 10 s per iteration
+    of the port on 16 threads); `rows` > 0 (--cpu-rows) overrides the rule."""
+    if rows > 0:
+        return min(cfg["n"], rows)
     k_mean = cfg["k"] if cfg["k"] else (cfg["kmax"] - cfg["kmin"]) / np.log(cfg["kmax"] / cfg["kmin"])
     if cfg["n"] * k_mean * cfg["r"] <= 1.0e11:
         return cfg["n"]
@@ -158,10 +182,12 @@ def prepare_cpu_sample(d, cfg, seed, rows):
     return rp, ci, va, m_s
 
 
-def run_cpu_baseline(sample, cfg, n, m, z, r, eps):
-    """Times one MU iteration of the port on the sample and scales each part by its own unit
-    count to the whole workload: the sparse products by entries, the H-sized dense parts by
-    columns, the W-sized ones by rows."""
+def run_cpu_baseline(sample, cfg, n, m, z, r, eps, iters=3):
+    """Times `iters` MU iterations of the port on the sample, one by one (the loss is not evaluated,
+    as the reference's own timer leaves it out, multi_mu_dense_factors_nmf1.h:188-200), and scales
+    each part by its own unit count to the whole workload: the sparse products by entries, the
+    H-sized dense parts by columns, the W-sized ones by rows.  `value` comes from the median
+    iteration; the fastest one is reported beside it."""
     from oracle import oracle as orc
 
     rp, ci, va, m_s = sample
@@ -173,26 +199,34 @@ def run_cpu_baseline(sample, cfg, n, m, z, r, eps):
     base = orc.F32Baseline(rp, ci, va, m_s, W0, eps=eps, Ht0_mr=Ht0)
     del Ht0
     threads = orc.F32Baseline.num_threads()
-    log(f"cpu baseline: context (host transposed CSR) in {time.perf_counter() - t0:.1f} s, {threads} threads, "
-        f"{cpu_model()}")
-    parts = base.step_timed(1)
-    base.close()
-    sample_s = sum(parts.values())
+    cores = physical_cores()
+    log(f"cpu baseline: context (host transposed CSR) in {time.perf_counter() - t0:.1f} s, {threads} threads on "
+        f"{cores} physical cores, {cpu_model()}")
     scale = {"spmm_n": z / z_s, "spmm_t": z / z_s, "gram_H": m / m_s, "xg_mu_H": m / m_s,
              "gram_W": n / n_s, "xg_mu_W": n / n_s}
-    full_s = sum(parts[k] * scale[k] for k in parts)
+    runs = []
+    for it in range(max(1, iters)):
+        parts = base.step_timed(1)
+        runs.append((sum(parts[k] * scale[k] for k in parts), sum(parts.values()), parts))
+        log(f"cpu baseline: iteration {it + 1} on the sample {runs[-1][1]:.2f} s -> {runs[-1][0]:.1f} s for the "
+            "whole workload; parts " + ", ".join(f"{k} {v:.2f}" for k, v in parts.items()))
+    base.close()
+    order = sorted(range(len(runs)), key=lambda i: runs[i][0])
+    full_s, sample_s, parts = runs[order[len(order) // 2]]  # the median iteration
+    best_s = runs[order[0]][0]
     whole = n_s == n
-    log(f"cpu baseline: one iteration on the sample {sample_s:.2f} s"
-        + ("" if whole else f" -> {full_s:.1f} s for the whole workload") + "; parts "
-        + ", ".join(f"{k} {v:.2f}" for k, v in parts.items()))
-    return {"value": 1.0 / full_s, "unit": "MU iterations/s", "cores": threads, "kind": "port",
-            "cpu_model": cpu_model(),
-            "sample": (f"1 MU iteration of the fp32 OpenMP port of the reference loop (loss excluded) on "
-                       + (f"the whole workload (n={n}, m={m}, nnz={z}, r={r})" if whole else
+    return {"value": 1.0 / full_s, "unit": "MU iterations/s", "cores": threads, "physical_cores": cores,
+            "kind": "port", "cpu_model": cpu_model(), "iterations_timed": len(runs),
+            "seconds_per_iteration_whole_workload": {"median": full_s, "min": best_s,
+                                                     "all": [x[0] for x in runs]},
+            "sample": (f"{len(runs)} MU iterations of the fp32 OpenMP port of the reference loop (loss excluded), "
+                       "timed one by one, on "
+                       + (f"the whole workload (n={n}, m={m}, nnz={z}, r={r}): median {full_s:.2f} s, fastest "
+                          f"{best_s:.2f} s" if whole else
                           f"the first {n_s} of {n} rows with their {m_s} non-empty columns ({z_s} entries, r={r}): "
-                          f"{sample_s:.2f} s; scaled to the whole workload part by part (sparse products by "
+                          f"median {sample_s:.2f} s; scaled to the whole workload part by part (sparse products by "
                           f"entries x{z / z_s:.1f}, H-sized parts by columns x{m / m_s:.2f}, W-sized by rows): "
-                          f"{full_s:.1f} s")),
+                          f"median {full_s:.1f} s, fastest {best_s:.1f} s")),
             "sample_seconds": sample_s, "parts_seconds_sample": parts}
 
 
@@ -292,7 +326,7 @@ def compare_decompositions(d, cfg, seed, r):
 
 def run_nmf(d, args, cfg):
     r = cfg["r"]
-    cpu_rows = cpu_sample_rows(cfg) if args.cpu_steps > 0 else 0
+    cpu_rows = cpu_sample_rows(cfg, args.cpu_rows) if args.cpu_steps > 0 else 0
     sample = prepare_cpu_sample(d, cfg, args.seed, cpu_rows) if 0 < cpu_rows < cfg["n"] else None
     comparison = (compare_decompositions(d, cfg, args.seed, r)
                   if cfg.get("compare_rows") and not args.no_compare else None)
@@ -391,10 +425,29 @@ def run_nmf(d, args, cfg):
 
     cpu_baseline = scipy_baseline = None
     if args.cpu_steps > 0:
-        cpu_baseline = run_cpu_baseline(sample, cfg, n, m, z, r, args.eps)
+        cpu_baseline = run_cpu_baseline(sample, cfg, n, m, z, r, args.eps, args.cpu_steps)
         if not args.no_scipy:
             scipy_baseline = run_scipy_baseline(sample, n, m, z, r, args.eps)
 
+    # The gather models beside the algorithmic bytes: what a product moves into the CUs when every
+    # gathered entry brings a whole row of a factor (4 r bytes).  "untiled": every entry of the matrix
+    # gathers; "planned": only the entries of the sparse part do, the dense head reads each of its
+    # factor rows once and its own block.  Rates are bytes over the measured time of the class, as a
+    # fraction of the HBM peak: above 1 means the caches served gathers, far below it with traffic near
+    # these bytes means the gathers went to the fabric.
+    P = 4 if z < 2**31 else 8
+    head_bytes = 4 * n_dense * (n + r)
+    gather_model = {}
+    for cls, ptr_bytes, streamed in (("spmm_n", P * (n + 1), 4 * n * r), ("spmm_t", P * (m + 1), 4 * n * r + 4 * r * m)):
+        if cls not in kernels:
+            continue
+        sec = kernels[cls]["ms"] / 1e3
+        untiled = 8 * z + ptr_bytes + 4 * r * z + (4 * n * r if cls == "spmm_n" else 4 * r * m)
+        planned = 8 * z_sparse + ptr_bytes + 4 * r * z_sparse + head_bytes + streamed
+        gather_model[cls] = {"bytes_untiled": untiled, "bytes_planned": planned,
+                             "untiled_frac_of_hbm_peak": untiled / sec / HBM_PEAK,
+                             "planned_frac_of_hbm_peak": planned / sec / HBM_PEAK,
+                             "planned_GBps": planned / sec / 1e9}
     out = {
         "metric": "NMF MU iterations/sec + SpMM achieved HBM GB/s (% of peak), 1 MI355X",
         "value": args.steps / elapsed,
@@ -415,6 +468,7 @@ def run_nmf(d, args, cfg):
                    "H_tile_columns": tile_cols, "device_memory_used_gb": (total - free1) / 1e9,
                    "device_memory_total_gb": total / 1e9},
         "roofline": roofline,
+        "roofline_gather_model": gather_model,
         "cpu_baseline": cpu_baseline,
         "cpu_baseline_scipy": scipy_baseline,
         "gpu_over_cpu": (args.steps / elapsed) / cpu_baseline["value"] if cpu_baseline else None,
@@ -581,8 +635,10 @@ def main():
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
     ap.add_argument("--eps", type=float, default=1e-12)
     ap.add_argument("--seed", type=int, default=43190432042)
-    ap.add_argument("--cpu-steps", type=int, default=1,
-                    help="0 skips the host-core baselines")
+    ap.add_argument("--cpu-steps", type=int, default=3,
+                    help="iterations of the host-core port that are timed (0 skips the host-core baselines)")
+    ap.add_argument("--cpu-rows", type=int, default=0,
+                    help="rows of the host-core sample (0 = about 10 s per iteration)")
     ap.add_argument("--fp32-steps", type=int, default=2,
                     help="steps timed with the matrix products on the fp32 matrix cores (0 = skip)")
     ap.add_argument("--no-scipy", action="store_true")

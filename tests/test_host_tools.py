@@ -233,3 +233,74 @@ def test_sparsify_d_npeff_feeds_the_fit(tmp_path):
     run("fit_coeffs_to_sparse_H", f"--output_path={fit}", f"--pef_path={pef}", f"--H_path={sparse}",
         "--n_splits_sparse_matmul=1", "--n_row_splits_pefs=1", "--nmf_max_iter=25", check=True)
     assert h5lite.read(fit, "data/W").shape == (n, r)
+
+
+@pytest.mark.gpu
+def test_run_nmf_on_pefs_at_a_realistic_size(tmp_path):
+    """configs[1] downscaled (1,000 examples x 16,384 values of 11M parameters, a 130 MB file made by
+    the device generator, rank 128, dense head and column panels in use): the executable's W, H and
+    reduce_kept_indices equal, bit for bit, those of the same fit driven through the C ABI."""
+    n, m_full, k, r, iters = 1000, 11_000_000, 16_384, 128, 10
+    pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=19, on_device=1)
+    assert os.path.getsize(pef) > 8 * n * k
+    out = str(tmp_path / "decomp.h5")
+    p = run("run_nmf_on_pefs", f"--output_path={out}", f"--per_example_fishers={pef}", f"--nmf_n_components={r}",
+            f"--nmf_max_iter={iters}", check=True)
+    lines = p.stdout.splitlines()
+    assert "Using 32 bit indices." in lines and "Running NMF using 32 bit indices." in lines
+    steps = [l for l in lines if l.startswith("step ")]
+    assert [s.split(":")[0] for s in steps] == ["step 10"]
+    vals, idx = h5lite.read(pef, "data/fisher/values"), h5lite.read(pef, "data/fisher/indices")
+    norms = h5lite.read(pef, "data/dense_fisher_norms")
+    A = d.Csr.from_pef(idx, vals, m_full)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=iters), consume_matrix=True)
+    hist = nmf.run(log=lambda s: None)
+    W, H, kept = h5lite.read(out, "data/W"), h5lite.read(out, "data/H"), h5lite.read(out, "data/reduce_kept_indices")
+    assert W.shape == (n, r) and H.shape == (r, A.n_cols) and A.n_cols > 1_000_000
+    assert np.array_equal(kept, A.kept_indices())
+    assert np.array_equal(W, nmf.loadWToHostSync()) and np.array_equal(H, nmf.loadHToHostSync())
+    logged = float(steps[-1].split(":")[1].split("[")[0])
+    assert abs(logged - hist[-1][1]) / hist[-1][1] < 1e-5
+    nmf.close()
+    A.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.timeout(1200)
+def test_wide_index_branch_from_a_file_past_int32(tmp_path):
+    """A PEF file with n_examples x n_fisher_values = 32,800 x 65,536 = 2,149,580,800 > INT32_MAX
+    (17 GB): the executable reads it with 64-bit indices (pef_fisher_h5.h:57-90); pruning the
+    parameters held by one example only brings the entries under INT32_MAX, so, by the
+    reference's rule, the factorisation is run and saved with IndT = int64
+    (run_nmf_on_pefs.cu:236-247, nmf_decomp_h5.h:58-75) without any override."""
+    import shutil
+
+    n, k, m_full, r = 32_800, 65_536, 110_000_000, 8
+    need_disk, need_ram = 30e9, 80e9
+    free_disk = shutil.disk_usage(str(tmp_path)).free
+    if free_disk < need_disk:
+        pytest.skip(f"needs {need_disk / 1e9:.0f} GB of scratch disk, {free_disk / 1e9:.0f} GB free")
+    ram = os.sysconf("SC_PAGE_SIZE") * os.sysconf("SC_AVPHYS_PAGES")
+    if ram < need_ram:
+        pytest.skip(f"needs {need_ram / 1e9:.0f} GB of free host memory, {ram / 1e9:.0f} GB available")
+    free, total = d.device_memory()
+    if free < 100e9:
+        pytest.skip("needs 100 GB of device memory")
+    pef = make_pef(tmp_path, n=n, m=m_full, k=k, seed=23, on_device=1)
+    assert os.path.getsize(pef) > 8 * n * k > 8 * 2**31
+    out = str(tmp_path / "wide.h5")
+    p = run("run_nmf_on_pefs", f"--output_path={out}", f"--per_example_fishers={pef}", f"--nmf_n_components={r}",
+            "--nmf_max_iter=2", "--min_values_per_parameter=2", check=True)
+    os.remove(pef)
+    lines = p.stdout.splitlines()
+    assert "Reading in PEFs using 64 bit indices." in lines
+    assert "Running NMF using 64 bit indices." in lines
+    kept = h5lite.read(out, "data/reduce_kept_indices")
+    fds, shape = h5lite.attr(out, "data/reduce_kept_indices", "full_dense_size")
+    assert kept.dtype == np.int64 and fds.dtype == np.int64 and shape == (1,) and int(fds[0]) == m_full
+    assert np.all(np.diff(kept) > 0) and 0 <= kept[0] and kept[-1] < m_full
+    W, H = h5lite.read(out, "data/W"), h5lite.read(out, "data/H")
+    assert W.shape == (n, r) and H.shape == (r, len(kept))
+    assert np.isfinite(W).all() and W.min() >= 0 and np.isfinite(H).all() and H.min() >= 0
