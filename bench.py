@@ -138,9 +138,11 @@ def price(cls, n, m, z, r, step_s, fused_gram, split_bf16):
 
 def traffic_from_profile(config, cls):
     """HBM-side bytes per MU iteration of a kernel class, read from the committed counter summary
-    profiles/nmf_<config>_hbm_traffic.md (a line `traffic_bytes <class> <bytes>`); (None, None)
+    profiles/nmf_<config>_hbm_traffic.md, or fit_<config>_hbm_traffic.md for the fit path (a line
+    `traffic_bytes <class> <bytes>`); (None, None)
     when there is no such file or line: counters cannot be read from inside this process."""
-    path = os.path.join(ROOT, "profiles", f"nmf_{config}_hbm_traffic.md")
+    kind = "fit" if CONFIGS.get(config, {}).get("kind") == "fit" else "nmf"
+    path = os.path.join(ROOT, "profiles", f"{kind}_{config}_hbm_traffic.md")
     try:
         for line in open(path):
             mm = re.match(r"\s*`?traffic_bytes\s+(\w+)\s+([0-9.eE+]+)`?", line)
@@ -615,7 +617,9 @@ def run_fit(d, args, cfg):
         "config": {"workload": cfg["name"], "n_examples": n, "n_features": m, "nnz_A": z, "nnz_per_row": cfg["k"],
                    "rank": r, "nnz_H": zh, "H_density": zh / (r * m), "eps": 1e-7, "seed": args.seed},
         "roofline": {"kernel": "k_spsp (A H^T of the first stage)", "bound": "hbm", "achieved": spsp_bytes / ah_s / 1e9,
-                     "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": spsp_bytes / ah_s / HBM_PEAK, "traffic": None},
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": spsp_bytes / ah_s / HBM_PEAK,
+                     "traffic": traffic_from_profile(args.config, "spsp_AHt")[0],
+                     "traffic_source": traffic_from_profile(args.config, "spsp_AHt")[1]},
         "first_stage": {"seconds_total": stage1_s, "AHt_ms": ah_s * 1e3, "HHt_ms": hh_s * 1e3,
                         "algorithmic_bytes": spsp_bytes},
         "second_stage": {"ms_per_step": ms_per_step, "hbm_frac": xg_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
