@@ -301,6 +301,14 @@ int dnpeff_nmf_loss_terms(dnpeff_nmf* nmf, double* sq_norm_A, double* pos, doubl
  * A H^T and one A^T W; does not change the factors. */
 int dnpeff_nmf_check_products(dnpeff_nmf* nmf, double* via_rows, double* via_columns);
 
+/* The sparseness projection of the columns of W that the reference builds for --sparsity_W and
+ * never runs: sparseContextW->sparsifyF() (dense_factor_sparsity_constraints.h:205-237; the one
+ * call, at multi_mu_dense_factors_nmf1.h:161-162, is commented out, and so no loop of this
+ * library calls it either).  l1_norm is FactorSparsenessConstraints::l1_norm (the flag's value),
+ * l2_norm its l2_norm (1 in the reference).  *rounds (may be NULL) receives the number of passes of
+ * its loop.  See dnpeff_op_sparsify_columns. */
+int dnpeff_nmf_sparsify_W(dnpeff_nmf* nmf, float l1_norm, float l2_norm, int* rounds);
+
 /* Copy the factors to the host in the output-file layout: W [n, r] row-major
  * (loadWToHostSync + toRowMajor_inPlace, nmf1.h:207-220, matrices.h:49-62),
  * H [r, m] row-major (loadHToHostSync + toRowMajor_inPlace, nmf1.h:222-240). */
@@ -369,6 +377,17 @@ int dnpeff_fit_destroy(dnpeff_fit* fit);
  * (cc/cuda_d_npeff/src/nmf/sparse/kernels.h:24-34) and
  * MultiplicativeUpdate_Kernel (nmf/kernels/mu.h:32-38). */
 int dnpeff_op_mu(int64_t count, float* F, const float* num, const float* den, float eps);
+
+/* Every column of the row-major factor W [n_rows, rank] is moved, in place, to non-negative
+ * entries that sum to l1_norm, by the iteration of DenseFactorSparsityContext::sparsifyF
+ * (dense_factor_sparsity_constraints.h:205-237) with the arithmetic of its kernels
+ * (sparsity_constraint_kernels.h:16-141): Hoyer's projection, except that the step length is the
+ * reference's expression (:51-65), which leaves ||column||^2 = l2_norm^2 + l1_norm^2 / (entries
+ * left non-zero) rather than l2_norm^2.  Column sums are taken in fp64 in a fixed order where the
+ * reference calls cublasSgemv / cublasSgemmStridedBatched (:405-452).  Synchronises once per pass
+ * (the reference's isFinishedSync, :363-374).  Fails for l1_norm <= 0 (a null constraint, :41-43). */
+int dnpeff_op_sparsify_columns(int64_t n_rows, int rank, float* W_nr, float l1_norm, float l2_norm,
+                               int* rounds);
 
 /* N[n, r] = A H^T with H given as [m, r].  cusparseSpMM(N, T) at
  * device_contexts1.h:255-258,317. */

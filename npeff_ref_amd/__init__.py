@@ -35,6 +35,7 @@ from .binding import (  # noqa: F401
     tuning_get,
     tuning_reset,
     op_mu,
+    op_sparsify_columns,
     op_spmm_n,
     op_threshold_compact,
     topk_rows,

@@ -97,6 +97,7 @@ SIGNATURES = {
     "dnpeff_nmf_loss": (C.c_int, [_p, C.POINTER(_f64)]),
     "dnpeff_nmf_loss_terms": (C.c_int, [_p, C.POINTER(_f64), C.POINTER(_f64), C.POINTER(_f64)]),
     "dnpeff_nmf_check_products": (C.c_int, [_p, C.POINTER(_f64), C.POINTER(_f64)]),
+    "dnpeff_nmf_sparsify_W": (C.c_int, [_p, _f32, _f32, C.POINTER(C.c_int)]),
     "dnpeff_nmf_get_W": (C.c_int, [_p, _p]),
     "dnpeff_nmf_get_H": (C.c_int, [_p, _p]),
     "dnpeff_nmf_device_factors": (C.c_int, [_p, _pp, _pp]),
@@ -112,6 +113,7 @@ SIGNATURES = {
     "dnpeff_fit_get_products": (C.c_int, [_p, _p, _p, C.POINTER(_f64)]),
     "dnpeff_fit_destroy": (C.c_int, [_p]),
     "dnpeff_op_mu": (C.c_int, [_i64, _p, _p, _p, _f32]),
+    "dnpeff_op_sparsify_columns": (C.c_int, [_i64, C.c_int, _p, _f32, _f32, C.POINTER(C.c_int)]),
     "dnpeff_op_spmm_n": (C.c_int, [_p, C.c_int, _p, _p]),
     "dnpeff_op_spmm_n_variant": (C.c_int, [_p, C.c_int, _p, _p, C.c_int]),
     "dnpeff_op_spmm_t": (C.c_int, [_p, C.c_int, _p, _p]),
@@ -287,6 +289,16 @@ class DeviceArray:
 
 def op_mu(F: DeviceArray, num: DeviceArray, den: DeviceArray, eps: float):
     _check(lib.dnpeff_op_mu(int(np.prod(F.shape)), F.ptr, num.ptr, den.ptr, eps))
+
+
+def op_sparsify_columns(W_nr: DeviceArray, l1_norm: float, l2_norm: float = 1.0) -> int:
+    """The reference's sparseness projection of every column of W [n, r], in place; returns the
+    number of passes of its loop (DenseFactorSparsityContext::sparsifyF,
+    dense_factor_sparsity_constraints.h:205-237)."""
+    rounds = C.c_int(0)
+    _check(lib.dnpeff_op_sparsify_columns(W_nr.shape[0], W_nr.shape[1], W_nr.ptr, l1_norm, l2_norm,
+                                          C.byref(rounds)))
+    return rounds.value
 
 
 def op_spmm_n(A: "Csr", r: int, H_mr: DeviceArray, N_nr: DeviceArray):
@@ -617,6 +629,13 @@ class MuNmf:
         a, b = _f64(0), _f64(0)
         _check(lib.dnpeff_nmf_check_products(self._h, C.byref(a), C.byref(b)))
         return a.value, b.value
+
+    def sparsify_W(self, l1_norm: float, l2_norm: float = 1.0) -> int:
+        """sparseContextW->sparsifyF() on the context's W (the call that the reference leaves
+        commented out at multi_mu_dense_factors_nmf1.h:161-162); returns the passes taken."""
+        rounds = C.c_int(0)
+        _check(lib.dnpeff_nmf_sparsify_W(self._h, l1_norm, l2_norm, C.byref(rounds)))
+        return rounds.value
 
     def loadWToHostSync(self) -> np.ndarray:
         """W as [n, r] row-major (after the reference's toRowMajor_inPlace)."""

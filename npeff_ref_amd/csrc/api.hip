@@ -543,6 +543,13 @@ DN_API int dnpeff_nmf_loss(dnpeff_nmf* nmf, double* out) {
   return 0;
 }
 
+DN_API int dnpeff_nmf_sparsify_W(dnpeff_nmf* nmf, float l1_norm, float l2_norm, int* rounds) {
+  clear_error();
+  DN_CHECK(nmf, "NULL argument");
+  // (H^T H and A H^T kept between calls depend on H only)
+  return sparsify_columns(nmf->n, nmf->r, nmf->W, l1_norm, l2_norm, rounds);
+}
+
 DN_API int dnpeff_nmf_get_W(dnpeff_nmf* nmf, float* W_nr) {
   clear_error();
   DN_CHECK(nmf && W_nr, "NULL argument");

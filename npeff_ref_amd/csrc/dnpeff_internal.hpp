@@ -143,6 +143,8 @@ int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr);
 int launch_spmm_n_reduce(const dnpeff_csr* A, int r, float* N_nr);
 int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 int launch_spsp(const dnpeff_csr* A, dnpeff_csr* B, float* partials);
+// sparsity.hip: the sparseness projection of the columns of a row-major [n, r] factor, in place
+int sparsify_columns(int64_t n, int r, float* W, float l1, float l2, int* rounds_out);
 int launch_chunk_reduce(const dnpeff_csr* A, int r, const float* partials, float* N_nr);
 
 // Switches for experiments and for tests that force a code path.  Each has an environment

@@ -24,7 +24,8 @@ struct ProgramFlags {
   std::string output_path, pef_path;
   int n_components = 0, max_iters = 0;
   int n_examples = -1, n_fisher_values = -1;
-  float sparsity_W = -1.0f;            // accepted, without effect (as in the reference)
+  float sparsity_W = -1.0f;            // accepted, without effect on the run (as in the reference, which
+                                       // never calls its projection; dnpeff_nmf_sparsify_W is that call)
   int min_values_per_parameter = 1;
   std::string initial_H_path, initial_W_path;  // accepted, without effect (as in the reference)
   // additions (optional): the reference hard-codes these at run_nmf_on_pefs.cu:189-192

@@ -31,6 +31,14 @@
  *                           monotonicity of the true loss.  The reference holds no
  *                           numeric fixture for these ("parity unpinned" against the
  *                           reference's own cuSPARSE/cuBLAS bits, by construction).
+ *   orc_sparsify_columns -- what its iteration fixes whatever the step length: every column
+ *                           ends non-negative with the prescribed sum, entries keep their
+ *                           order, a column that needs no second pass is an affine image of
+ *                           its input; and what the reference's step length fixes:
+ *                           ||column||^2 = l2^2 + l1^2 / (entries left non-zero), against l2^2
+ *                           for Hoyer's own (tests/test_oracle_sparsify.py).  The reference
+ *                           never runs this code and holds no vector for it: "parity
+ *                           unpinned" against the reference's bits.
  */
 #include <math.h>
 #include <stdint.h>
@@ -805,6 +813,69 @@ ORC_API void orc_f32_destroy(void* ctx) {
   free(c->colptr); free(c->rowind); free(c->tvals);
   free(c->W); free(c->Ht); free(c->num); free(c->G);
   free(c);
+}
+
+/* The sparseness projection of the columns of a row-major factor W [n, r], in place; returns the
+ * largest number of passes any column took.  One column at a time (the reference steps all
+ * columns together and leaves those without negative entries alone: the same values).
+ * DenseFactorSparsityContext::sparsifyF, cc/cuda_d_npeff/src/nmf/sparse/
+ * dense_factor_sparsity_constraints.h:205-237; element arithmetic of
+ * sparsity_constraint_kernels.h:16-141 in fp32; the column sums (cublasSgemv /
+ * cublasSgemmStridedBatched there, :405-452) in fp64, rounded to fp32. */
+ORC_API int orc_sparsify_columns(int64_t n, int r, float* W, float l1, float l2) {
+  int most = 0;
+  float* s = (float*)malloc(sizeof(float) * (size_t)n);
+  float* y = (float*)malloc(sizeof(float) * (size_t)n);
+  for (int c = 0; c < r; c++) {
+    double acc = 0.0;
+    for (int64_t i = 0; i < n; i++) { s[i] = W[i * r + c]; y[i] = 1.0f; acc += (double)s[i]; } /* :240-257 */
+    const float sum_x = (float)acc;
+    for (int64_t i = 0; i < n; i++) s[i] += (l1 - sum_x) / (float)n; /* kernel_computeInitialS :16-27 */
+    int passes = 0;
+    for (;;) {
+      passes++;
+      double yy_d = 0.0, ss_d = 0.0, sy_d = 0.0; /* :222, :281-286 */
+      for (int64_t i = 0; i < n; i++) {
+        yy_d += (double)y[i];
+        ss_d += (double)(s[i] * s[i]);
+        sy_d += (double)(s[i] * y[i]);
+      }
+      const float YY = (float)yy_d, SS = (float)ss_d, SY = (float)sy_d;
+      /* kernel_computeAlpha :41-66 */
+      const float L2 = sqrtf(l2 * l2);
+      const float beta = l1 / YY;
+      const float m2 = beta * beta * YY;
+      const float ms = beta * SY;
+      const float m_s_2 = fmaxf(1e-9f, beta * beta * YY + SS - 2.0f * beta * SY);
+      const float alpha = (L2 * sqrtf(m_s_2) + m2 - ms) / m_s_2;
+      /* kernel_updateSAfterAlpha :69-88 */
+      int64_t negative = 0;
+      for (int64_t i = 0; i < n; i++) {
+        const float m = y[i] * l1 / YY;
+        const float v = m + alpha * (s[i] - m);
+        s[i] = v;
+        negative += v < 0.0f;
+      }
+      if (negative == 0) break; /* :352-374 */
+      /* kernel_updateYAndS :91-113 */
+      for (int64_t i = 0; i < n; i++) {
+        if (y[i] != 0.0f && s[i] < 0.0f) y[i] = 0.0f;
+        if (y[i] == 0.0f) s[i] = 0.0f;
+      }
+      /* kernel_updateSLastStep :116-141 with the sums of :391-392 */
+      double sum_s = 0.0, sum_y = 0.0;
+      for (int64_t i = 0; i < n; i++) { sum_s += (double)s[i]; sum_y += (double)y[i]; }
+      const float cshift = ((float)sum_s - l1) / (float)sum_y;
+      for (int64_t i = 0; i < n; i++)
+        if (y[i] != 0.0f) s[i] -= cshift;
+      if (passes > n + 1) break; /* cannot happen: every pass fixes one more entry at zero */
+    }
+    for (int64_t i = 0; i < n; i++) W[i * r + c] = s[i];
+    if (passes > most) most = passes;
+  }
+  free(s);
+  free(y);
+  return most;
 }
 
 ORC_API int orc_num_threads(void) {

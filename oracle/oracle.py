@@ -62,6 +62,7 @@ _f32_fit_timed = _sig(_lib, "orc_f32_fit_steps_timed", _f64, [_i64, C.c_int, _p,
 _f32_get = _sig(_lib, "orc_f32_get", None, [_p, _p, _p])
 _f32_destroy = _sig(_lib, "orc_f32_destroy", None, [_p])
 _num_threads = _sig(_lib, "orc_num_threads", C.c_int, [])
+_sparsify_cols = _sig(_lib, "orc_sparsify_columns", C.c_int, [_i64, C.c_int, _p, _f32, _f32])
 
 
 def _csr(rowptr, colind, vals):
@@ -314,6 +315,14 @@ def sparsify_H(W, H_rm, threshold):
         W2[:, k] *= div
     return (W2, np.concatenate(vals).astype(np.float32), np.array(offs, dtype=np.int64),
             np.concatenate(cols).astype(np.int32))
+
+
+def sparsify_columns(W, l1_norm, l2_norm=1.0):
+    """(W', passes): every column of the row-major W moved to non-negative entries that sum to
+    l1_norm by the reference's iteration (dense_factor_sparsity_constraints.h:205-237)."""
+    out = np.array(W, dtype=np.float32, order="C", copy=True)
+    passes = _sparsify_cols(out.shape[0], out.shape[1], _ptr(out), l1_norm, l2_norm)
+    return out, passes
 
 
 def topk_rows(x, k):
