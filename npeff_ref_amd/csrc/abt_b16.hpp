@@ -163,4 +163,99 @@ __device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, in
   }
 }
 
+// A diagonal tile of X^T X (128 columns of X against themselves) with the work that its symmetry
+// leaves: of the 4 x 4 blocks of 32 x 32 only the ten with block row <= block column are formed,
+// and a block on the diagonal needs four of the six partial products, because h^T m and m^T h
+// (and h^T l, l^T h) are transposes of each other there:
+//   G_bb = Q + P + P^T,  Q = h^T h + m^T m,  P = h^T m + h^T l.
+// Waves 0 and 1 take the block pairs (0, 1) and (2, 3): the block between the two (six products)
+// and the two diagonal blocks (Q and P apart, two products each): 14 matrix instructions per 16
+// contraction elements.  Waves 2 and 3 take blocks (0, 2), (0, 3) and (1, 2), (1, 3): 12.  (All
+// sixteen blocks with six products are 24 per wave.)  The operand tile is fetched, split and
+// stored once; a block row of it serves as first and as second operand alike (both are read as
+// [row][8 contraction elements per half wave]).
+// acc: pair waves: [0] = block (p, p + 1), [1] = Q_p, [2] = P_p, [3] = Q_p+1, [4] = P_p+1 with
+// p = 2 wave; the others: [0] = block (a, 2), [1] = block (a, 3) with a = wave - 2.
+template <int STAGES>
+__device__ __forceinline__ void gram_diag_mainloop(const float* __restrict__ src, int64_t ld,
+                                                   int64_t first, int64_t stride, int64_t n_tiles,
+                                                   unsigned char* ab, abt_acc16 (&acc)[5]) {
+  static_assert(STAGES == 1 || STAGES == 2, "one or two tiles in registers");
+  if (n_tiles <= 0) return;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l32 = lane & 31, half = lane >> 5;
+  const bool pair = wave < 2;
+  AbtOperand<true> oa[STAGES];
+  auto fetch = [&](int s, int64_t t) {
+    const int64_t k0 = (first + (t < n_tiles ? t : n_tiles - 1) * stride) * ABT_KB;
+    oa[s].fetch(src, ld, k0);
+  };
+  const unsigned char* lane_at = ab + l32 * ABT_LD + 16 * half;
+  const unsigned char* row_x = lane_at + 32 * (pair ? 2 * wave : wave - 2) * ABT_LD;
+  const unsigned char* row_y = lane_at + 32 * (pair ? 2 * wave + 1 : 2) * ABT_LD;
+  const unsigned char* row_w = lane_at + 32 * 3 * ABT_LD;
+  auto planes = [&](const unsigned char* p, bf16x8& h, bf16x8& m, bf16x8& l) {
+    h = *reinterpret_cast<const bf16x8*>(p);
+    m = *reinterpret_cast<const bf16x8*>(p + ABT_PLANE);
+    l = *reinterpret_cast<const bf16x8*>(p + 2 * ABT_PLANE);
+  };
+  auto mfma_tile = [&]() {
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+      bf16x8 xh, xm, xl, yh, ym, yl;
+      planes(row_x + 32 * st, xh, xm, xl);
+      planes(row_y + 32 * st, yh, ym, yl);
+      if (pair) {
+        // the six products of the block between alternate with the eight of the diagonal blocks
+        acc[0] = DN_MFMA_B16(xh, yh, acc[0]);
+        acc[1] = DN_MFMA_B16(xh, xh, acc[1]);
+        acc[0] = DN_MFMA_B16(xh, ym, acc[0]);
+        acc[3] = DN_MFMA_B16(yh, yh, acc[3]);
+        acc[0] = DN_MFMA_B16(xm, yh, acc[0]);
+        acc[2] = DN_MFMA_B16(xh, xm, acc[2]);
+        acc[0] = DN_MFMA_B16(xh, yl, acc[0]);
+        acc[4] = DN_MFMA_B16(yh, ym, acc[4]);
+        acc[0] = DN_MFMA_B16(xl, yh, acc[0]);
+        acc[1] = DN_MFMA_B16(xm, xm, acc[1]);
+        acc[0] = DN_MFMA_B16(xm, ym, acc[0]);
+        acc[3] = DN_MFMA_B16(ym, ym, acc[3]);
+        acc[2] = DN_MFMA_B16(xh, xl, acc[2]);
+        acc[4] = DN_MFMA_B16(yh, yl, acc[4]);
+      } else {
+        bf16x8 wh, wm, wl;
+        planes(row_w + 32 * st, wh, wm, wl);
+        acc[0] = DN_MFMA_B16(xh, yh, acc[0]);
+        acc[1] = DN_MFMA_B16(xh, wh, acc[1]);
+        acc[0] = DN_MFMA_B16(xh, ym, acc[0]);
+        acc[1] = DN_MFMA_B16(xh, wm, acc[1]);
+        acc[0] = DN_MFMA_B16(xm, yh, acc[0]);
+        acc[1] = DN_MFMA_B16(xm, wh, acc[1]);
+        acc[0] = DN_MFMA_B16(xh, yl, acc[0]);
+        acc[1] = DN_MFMA_B16(xh, wl, acc[1]);
+        acc[0] = DN_MFMA_B16(xl, yh, acc[0]);
+        acc[1] = DN_MFMA_B16(xl, wh, acc[1]);
+        acc[0] = DN_MFMA_B16(xm, ym, acc[0]);
+        acc[1] = DN_MFMA_B16(xm, wm, acc[1]);
+      }
+    }
+  };
+  fetch(0, 0);
+  oa[0].commit(ab);
+#pragma unroll
+  for (int s = 0; s < STAGES; s++) fetch((1 + s) % STAGES, 1 + s);
+  __syncthreads();
+  for (int64_t t = 0; t < n_tiles; t += STAGES) {
+#pragma unroll
+    for (int u = 0; u < STAGES; u++) {
+      if (t + u < n_tiles) {
+        mfma_tile();
+        __syncthreads();  // every wave is done with the planes
+        oa[(u + 1) % STAGES].commit(ab);
+        fetch((u + 1) % STAGES, t + u + 1 + STAGES);
+        __syncthreads();
+      }
+    }
+  }
+}
+
 }  // namespace dn

@@ -170,6 +170,7 @@ struct tuning_t {
   double nl_piece_cols = 16384.0;  // columns per piece of the slot lists
   double nl_lag = 1.0;             // pieces the workgroups of an XCD may be apart
   double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
+  double gram_fold = 1.0;          // diagonal tiles of X^T X with the work their symmetry leaves (0 = all sixteen blocks)
   double nl_wgs = 64.0;            // workgroups of the slot-list kernel per XCD (two per CU)
   double nl_spin = 50000.0;        // polls (about 1 us each) before a workgroup of the slot-list kernel stops waiting
   double verbose = 0.0;

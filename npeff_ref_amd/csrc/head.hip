@@ -362,7 +362,7 @@ int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
 // one more term of every tile (the last rows, from the fp32 kernel).
 __global__ void __launch_bounds__(256)
     k_gram_tiles_reduce(const float* __restrict__ ws, int64_t s_diag, int64_t s_off, int64_t extra, int r,
-                        float* __restrict__ G) {
+                        bool folded, float* __restrict__ G) {
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= r * r) return;
   const int a = e / r, b = e % r;
@@ -370,6 +370,12 @@ __global__ void __launch_bounds__(256)
   double s = 0.0;
   const int64_t stride = (int64_t)r * r;
   const int64_t slices = (a >> 7) == (b >> 7) ? s_diag : s_off;
+  if (folded && (a >> 5) == (b >> 5)) {
+    // a diagonal block of 32 x 32 from k_gram_diag_b16: the stored block plus its transpose
+    const int et = b * r + a;
+    for (int64_t sl = 0; sl < slices; sl++)
+      s += (double)ws[sl * stride + e] + (double)ws[sl * stride + et];
+  } else
   for (int64_t sl = 0; sl < slices; sl++) s += (double)ws[sl * stride + e];
   if (extra >= 0) s += (double)ws[extra * stride + e];
   G[(int64_t)a * r + b] = (float)s;
@@ -420,9 +426,50 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         base[(int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * r + 32 * j] = acc[i][j][v];
 }
 
+// The diagonal tiles with the work their symmetry leaves (gram_diag_mainloop): the ten upper
+// blocks of 32 x 32 are stored, those on the diagonal as Q / 2 + P, so that the reduction gets
+// Q + P + P^T as the sum of the stored block and its transpose.
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_gram_diag_b16(const float* __restrict__ X, int64_t k_tiles, int r, float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char ab[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int ti = blockIdx.x;
+  const int64_t S = gridDim.z, z = blockIdx.z;
+  const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
+  acc16 acc[5];
+#pragma unroll
+  for (int b = 0; b < 5; b++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[b][v] = 0.0f;
+  gram_diag_mainloop<ABT_STAGES_GRAM>(X + 128 * ti, r, z, S, n_my, ab, acc);
+  float* tile = out + ((int64_t)z * r + 128 * ti + 4 * half) * r + 128 * ti + l32;
+  auto store = [&](int bi, int bj, const acc16& c) {
+    float* base = tile + (int64_t)(32 * bi) * r + 32 * bj;
+#pragma unroll
+    for (int v = 0; v < 16; v++) base[(int64_t)(8 * (v >> 2) + (v & 3)) * r] = c[v];
+  };
+  if (wave < 2) {
+    const int p = 2 * wave;
+    store(p, p + 1, acc[0]);
+    acc16 d0, d1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      d0[v] = 0.5f * acc[1][v] + acc[2][v];
+      d1[v] = 0.5f * acc[3][v] + acc[4][v];
+    }
+    store(p, p, d0);
+    store(p + 1, p + 1, d1);
+  } else {
+    store(wave - 2, 2, acc[0]);
+    store(wave - 2, 3, acc[1]);
+  }
+}
+
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace) {
   const int t = r / 128;
   int64_t s_diag, s_off, extra = -1;
+  bool folded = false;
   if (use_split_bf16() && rows >= ABT_KB) {
     static bool attr_set = false;
     if (!attr_set) {
@@ -430,14 +477,21 @@ int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* work
                                  hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
       DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_tiles_b16<false>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+      DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_diag_b16),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
       attr_set = true;
     }
     // whole contraction tiles on the bf16 matrix cores, the last rows (fewer than 32) as one
     // more slice through the fp32 kernel
     const int64_t k_tiles = rows / ABT_KB, whole = k_tiles * ABT_KB;
     gram_b16_slices(rows, r, &s_diag, &s_off);
-    hipLaunchKernelGGL(k_gram_tiles_b16<true>, dim3((unsigned)t, 1, (unsigned)s_diag), dim3(256), ABT_LDS,
-                       stream(), X, k_tiles, r, t, workspace);
+    folded = tuning().gram_fold != 0;
+    if (folded)
+      hipLaunchKernelGGL(k_gram_diag_b16, dim3((unsigned)t, 1, (unsigned)s_diag), dim3(256), ABT_LDS, stream(),
+                         X, k_tiles, r, workspace);
+    else
+      hipLaunchKernelGGL(k_gram_tiles_b16<true>, dim3((unsigned)t, 1, (unsigned)s_diag), dim3(256), ABT_LDS,
+                         stream(), X, k_tiles, r, t, workspace);
     if (t > 1)
       hipLaunchKernelGGL(k_gram_tiles_b16<false>, dim3((unsigned)(t * (t - 1) / 2), 1, (unsigned)s_off),
                          dim3(256), ABT_LDS, stream(), X, k_tiles, r, t, workspace);
@@ -452,7 +506,7 @@ int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* work
     DN_TRY(launch_ptq(X, r, rows, X, r, r, r, s_diag, workspace, t));
   }
   hipLaunchKernelGGL(k_gram_tiles_reduce, dim3((unsigned)ceil_div((int64_t)r * r, 256)), dim3(256), 0,
-                     stream(), workspace, s_diag, s_off, extra, r, G);
+                     stream(), workspace, s_diag, s_off, extra, r, folded, G);
   DN_LAUNCH_CHECK();
   return 0;
 }

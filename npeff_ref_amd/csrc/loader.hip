@@ -99,6 +99,7 @@ static const tuning_entry g_tuning_table[] = {
     {"nl_piece_cols", &tuning_t::nl_piece_cols}, {"nl_lag", &tuning_t::nl_lag},
     {"nl_spin", &tuning_t::nl_spin},             {"nl_wgs", &tuning_t::nl_wgs},
     {"gram_beside", &tuning_t::gram_beside},
+    {"gram_fold", &tuning_t::gram_fold},
 };
 
 static tuning_t tuning_from_env() {

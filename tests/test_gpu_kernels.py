@@ -84,6 +84,26 @@ def test_gram(rows, r):
     assert np.array_equal(G, G.T) or _rel(G, G.T.astype(np.float64)) < 1e-6
 
 
+@pytest.mark.parametrize("fold", [1, 0])
+@pytest.mark.parametrize("rows,r", [(4096, 256), (20011, 256), (3000, 384), (2500, 1024)])
+def test_gram_diagonal_tiles_with_and_without_their_symmetry(rows, r, fold, tune):
+    """X^T X at the ranks that run on tiles, with signed entries over eight decades (a partial
+    product taken from the wrong side of the diagonal, or left out, shows at 2^-8 or 2^-16 of the
+    element), the diagonal tiles folded (ten blocks, four products on the diagonal ones) and not."""
+    tune("gram_fold", fold)
+    rng = np.random.default_rng(rows + r + fold)
+    X = (rng.standard_normal((rows, r)) * 10.0 ** rng.uniform(-4, 4, size=(1, r))).astype(np.float32)
+    dG = d.DeviceArray((r, r))
+    d.op_gram(d.DeviceArray.from_numpy(X), dG)
+    G = dG.numpy()
+    want = orc.gram_f64(X)
+    scale = np.sqrt(np.outer(np.diag(want), np.diag(want)))  # |G_ab| <= sqrt(G_aa G_bb)
+    assert np.all(np.abs(G - want) <= 2e-6 * scale)
+    assert np.array_equal(G, G.T)
+    d.op_gram(d.DeviceArray.from_numpy(X), dG)
+    assert np.array_equal(dG.numpy(), G)
+
+
 @pytest.mark.parametrize("rows,r", [(1, 16), (33, 16), (1000, 50), (4100, 128), (5000, 256), (3000, 512), (300, 130),
                                     (700, 64), (1000, 100), (513, 36), (300, 20), (257, 32), (70001, 128),
                                     (140000, 64), (256, 128), (255, 128), (1001, 384), (40000, 256), (257, 1024)])
