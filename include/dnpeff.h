@@ -77,7 +77,8 @@ int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int
 /* Switches for experiments and for tests that must reach a particular code path; no counterpart
  * in the reference.  Names: dense_fill, panels, sweep_bytes, sweep_min, sweep_waves, sweep_lag,
  * sweep_spin, spmm_t_slices, split_bf16, fused_gram, h_tile_mb, tiled_h, topk_fast_cap, verbose,
- * gram_beside (H^T H of the W update on a second stream beside A H^T), n_lists, t_lists (the sparse
+ * gram_beside (H^T H of the W update on a second stream beside A H^T), gram_fold (0: diagonal
+ * tiles of X^T X without the use of their symmetry), n_lists, t_lists (the sparse
  * products on component slices of 32: slot lists / column blocks), nl_piece_cols, nl_lag, nl_spin,
  * nl_wgs (their piece size, lock step and launch shape).
  * Each starts from the environment variable DNPEFF_<NAME IN CAPITALS> (read once, when the
