@@ -1,5 +1,6 @@
 // Handles of the two hot loops behind the C ABI: the dense-factor MU NMF of
 // run_nmf_on_pefs and the W-only learner of fit_coeffs_to_sparse_H.
+#include <chrono>
 #include "dnpeff_internal.hpp"
 
 #include <algorithm>
@@ -267,17 +268,31 @@ static int nmf_create_impl(dnpeff_csr* A, int rank, float eps, int64_t seed, uns
   // multi_mu_dense_factors_nmf1.h:95-99
   DN_CHECK(A->n_rows <= A->n_cols, "Error: Not handling matrices with more rows than columns yet.");
   const bool consume = (flags & DNPEFF_NMF_CONSUME_MATRIX) != 0;
+  // with verbose set: seconds of each phase of the set-up (the stream is drained at every mark)
+  const bool timed = tuning().verbose != 0.0;
+  auto t_last = std::chrono::steady_clock::now();
+  auto mark = [&](const char* what) {
+    if (!timed) return;
+    (void)hipStreamSynchronize(stream());
+    const auto t = std::chrono::steady_clock::now();
+    fprintf(stderr, "dnpeff: set-up: %-44s %7.3f s\n", what, std::chrono::duration<double>(t - t_last).count());
+    t_last = t;
+  };
   double sq_norm = 0.0;
   DN_TRY(dnpeff_csr_sq_norm(A, &sq_norm));
+  mark("||A||^2");
   bool tiled = false;
   DN_TRY(plan_matrix(A, rank, consume, &tiled));
+  mark("memory plan, dense head and sparse tail");
   if (consume && A->tail) {  // the tail and the head hold everything the products read
     DN_HIP(hipStreamSynchronize(stream()));
     dfree(A->colind); A->colind = nullptr;
     dfree(A->vals); A->vals = nullptr;
   }
   DN_TRY(csr_ensure_products(A, rank));
+  mark("transposed copy, panels, pieces, work lists");
   if (consume) DN_TRY(csr_consume_for_products(A));
+  mark("release of what the products do not read");
   dnpeff_nmf* h = new dnpeff_nmf();
   h->A = A; h->r = rank; h->eps = eps; h->seed = (uint64_t)seed;
   h->n = A->n_rows; h->m = A->n_cols;
@@ -299,6 +314,7 @@ static int nmf_create_impl(dnpeff_csr* A, int rank, float eps, int64_t seed, uns
     s = dmalloc(&h->GH, (int64_t)rank * rank) || dmalloc(&h->gpart, xg_mu_gram_workspace_floats(h->m));
   if (!s && h->tiled) s = csr_tile_lists(A);
   if (s) { dnpeff_nmf_destroy(h); return s; }
+  mark("factors and workspaces");
   if (tuning().verbose != 0.0) {
     size_t free_b = 0, total_b = 0;
     (void)hipMemGetInfo(&free_b, &total_b);
