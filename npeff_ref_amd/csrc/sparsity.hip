@@ -25,17 +25,18 @@
 
 namespace dn {
 
-constexpr int HOYER_ROWS = 32;  // rows of W per workgroup in the passes that sum
+constexpr int HOYER_ROWS = 32;      // rows of W per workgroup in the passes that sum, at least
+constexpr int HOYER_BLOCKS = 4096;  // and at most this many workgroups (partial sums per column)
 
 // part[b][q][c] = sums over the rows of block b:  MODE 0: q0 = sum S
 // MODE 1: q0 = sum Y, q1 = sum S S, q2 = sum S Y
 // MODE 3 (after fixing the negative entries of active columns at zero): q0 = sum S, q1 = sum Y
 template <int MODE>
 __global__ void __launch_bounds__(256)
-    k_hoyer_sums(int64_t n, int r, float* __restrict__ S, unsigned char* __restrict__ Y,
+    k_hoyer_sums(int64_t n, int r, int64_t per, float* __restrict__ S, unsigned char* __restrict__ Y,
                  const float* __restrict__ active, double* __restrict__ part) {
-  const int64_t row0 = (int64_t)blockIdx.x * HOYER_ROWS;
-  const int64_t row1 = row0 + HOYER_ROWS < n ? row0 + HOYER_ROWS : n;
+  const int64_t row0 = (int64_t)blockIdx.x * per;
+  const int64_t row1 = row0 + per < n ? row0 + per : n;
   for (int c = threadIdx.x; c < r; c += 256) {
     double q0 = 0.0, q1 = 0.0, q2 = 0.0;
     const bool act = MODE == 3 ? active[c] != 0.0f : true;
@@ -123,11 +124,11 @@ __global__ void __launch_bounds__(256)
 // kernel_updateSAfterAlpha (:69-88) on the active columns, and the number of negative entries
 // that it leaves in the rows of this block: neg[b][c] (0 for a column that is not active)
 __global__ void __launch_bounds__(256)
-    k_hoyer_step(int64_t n, int r, float* __restrict__ S, const unsigned char* __restrict__ Y,
+    k_hoyer_step(int64_t n, int r, int64_t per, float* __restrict__ S, const unsigned char* __restrict__ Y,
                  const float* __restrict__ alpha, const float* __restrict__ yy,
                  const float* __restrict__ active, float l1, int* __restrict__ neg) {
-  const int64_t row0 = (int64_t)blockIdx.x * HOYER_ROWS;
-  const int64_t row1 = row0 + HOYER_ROWS < n ? row0 + HOYER_ROWS : n;
+  const int64_t row0 = (int64_t)blockIdx.x * per;
+  const int64_t row1 = row0 + per < n ? row0 + per : n;
   for (int c = threadIdx.x; c < r; c += 256) {
     int count = 0;
     if (active[c] != 0.0f) {
@@ -177,7 +178,8 @@ __global__ void k_hoyer_fill(int r, float* active, int* any) {
 int sparsify_columns(int64_t n, int r, float* W, float l1, float l2, int* rounds_out) {
   DN_CHECK(n >= 1 && r >= 1 && r <= (1 << 20), "sparsify: %lld rows, rank %d", (long long)n, r);
   DN_CHECK(l1 > 0.0f, "sparsify: l1 norm %g is not positive (a null constraint)", (double)l1);
-  const int64_t blocks = ceil_div(n, HOYER_ROWS), total = n * r;
+  const int64_t per = std::max<int64_t>(HOYER_ROWS, ceil_div(n, HOYER_BLOCKS));
+  const int64_t blocks = ceil_div(n, per), total = n * r;
   dbuf<unsigned char> Y;
   dbuf<double> part;
   dbuf<float> coef, yy, active;
@@ -193,7 +195,7 @@ int sparsify_columns(int64_t n, int r, float* W, float l1, float l2, int* rounds
   const dim3 g_flat((unsigned)std::min<int64_t>(ceil_div(total, 256), 65536));
   hipStream_t st = stream();
   hipLaunchKernelGGL(k_hoyer_fill, g_r, b256, 0, st, r, active.p, any.p);
-  hipLaunchKernelGGL(k_hoyer_sums<0>, g_rows, b256, 0, st, n, r, W, Y.p, active.p, part.p);
+  hipLaunchKernelGGL(k_hoyer_sums<0>, g_rows, b256, 0, st, n, r, per, W, Y.p, active.p, part.p);
   hipLaunchKernelGGL(k_hoyer_coef<0>, g_r, b256, 0, st, n, r, blocks, part.p, l1, l2, coef.p, yy.p);
   hipLaunchKernelGGL(k_hoyer_start, g_flat, b256, 0, st, total, r, W, Y.p, coef.p);
   DN_LAUNCH_CHECK();
@@ -201,9 +203,9 @@ int sparsify_columns(int64_t n, int r, float* W, float l1, float l2, int* rounds
   int rounds = 0;
   for (;; rounds++) {
     DN_CHECK(rounds <= n, "sparsify: no end after %d rounds", rounds);
-    hipLaunchKernelGGL(k_hoyer_sums<1>, g_rows, b256, 0, st, n, r, W, Y.p, active.p, part.p);
+    hipLaunchKernelGGL(k_hoyer_sums<1>, g_rows, b256, 0, st, n, r, per, W, Y.p, active.p, part.p);
     hipLaunchKernelGGL(k_hoyer_coef<1>, g_r, b256, 0, st, n, r, blocks, part.p, l1, l2, coef.p, yy.p);
-    hipLaunchKernelGGL(k_hoyer_step, g_rows, b256, 0, st, n, r, W, Y.p, coef.p, yy.p, active.p, l1, neg.p);
+    hipLaunchKernelGGL(k_hoyer_step, g_rows, b256, 0, st, n, r, per, W, Y.p, coef.p, yy.p, active.p, l1, neg.p);
     hipLaunchKernelGGL(k_hoyer_mask, g_r, b256, 0, st, r, blocks, neg.p, active.p, any.p);
     DN_LAUNCH_CHECK();
     int host_any = 0;
@@ -211,7 +213,7 @@ int sparsify_columns(int64_t n, int r, float* W, float l1, float l2, int* rounds
     DN_HIP(hipStreamSynchronize(st));
     if (!host_any) break;
     hipLaunchKernelGGL(k_hoyer_fill, dim3(1), dim3(1), 0, st, 0, active.p, any.p);  // any = 0
-    hipLaunchKernelGGL(k_hoyer_sums<3>, g_rows, b256, 0, st, n, r, W, Y.p, active.p, part.p);
+    hipLaunchKernelGGL(k_hoyer_sums<3>, g_rows, b256, 0, st, n, r, per, W, Y.p, active.p, part.p);
     hipLaunchKernelGGL(k_hoyer_coef<3>, g_r, b256, 0, st, n, r, blocks, part.p, l1, l2, coef.p, yy.p);
     hipLaunchKernelGGL(k_hoyer_shift, g_flat, b256, 0, st, total, r, W, Y.p, coef.p, active.p);
     DN_LAUNCH_CHECK();

@@ -26,7 +26,7 @@ def _compare(got, want, l1):
 
 
 @pytest.mark.parametrize("n,r,l1", [(1, 1, 1.0), (2, 1, 1.0), (37, 5, 2.0), (500, 8, 5.0), (2000, 256, 12.0),
-                                    (4099, 100, 30.0), (300, 1000, 4.0), (20000, 256, 40.0)])
+                                    (4099, 100, 30.0), (300, 1000, 4.0), (20000, 256, 40.0), (300001, 3, 60.0)])
 def test_columns_match_the_oracle(n, r, l1):
     rng = np.random.default_rng(n + r)
     W = (rng.random((n, r)) ** 2).astype(np.float32)
