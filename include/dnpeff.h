@@ -175,6 +175,12 @@ int dnpeff_csr_split_dense_head(dnpeff_csr* A, double min_fill, int64_t* n_dense
 /* Columns in the dense head (0 = not split) and entries left in the sparse part. */
 int dnpeff_csr_head_info(const dnpeff_csr* A, int64_t* n_dense, int64_t* nnz_sparse);
 
+/* How the sparse part is organised for A H^T once a product or a context has planned it:
+ * out6 = column panels, of which plain, swept pieces, first column of the far tail that runs from
+ * slot lists (0 = none), entries and batches of 64 in the slot lists (0 = none).  No counterpart in
+ * the reference (cusparseSpMM_preprocess, device_contexts1.h:255-265, keeps its plan to itself). */
+int dnpeff_csr_products_info(const dnpeff_csr* A, int64_t* out6);
+
 /* Copy the transposed CSR back: colptr[n_cols+1], rowind[nnz], vals[nnz]. */
 int dnpeff_csr_download_transpose(dnpeff_csr* A, int64_t* colptr, int32_t* rowind, float* vals);
 

@@ -69,6 +69,7 @@ SIGNATURES = {
     "dnpeff_op_threshold_compact": (C.c_int, [C.c_int64, _p, C.c_float, C.c_float, _p, _p, C.POINTER(C.c_int64)]),
     "dnpeff_csr_split_dense_head": (C.c_int, [_p, C.c_double, C.POINTER(C.c_int64)]),
     "dnpeff_csr_head_info": (C.c_int, [_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "dnpeff_csr_products_info": (C.c_int, [_p, _p]),
     "dnpeff_csr_download_transpose": (C.c_int, [_p, _p, _p, _p]),
     "dnpeff_csr_release": (C.c_int, [_p, C.c_int]),
     "dnpeff_csr_destroy": (C.c_int, [_p]),
@@ -504,6 +505,13 @@ class Csr:
         nd, zs = _i64(0), _i64(0)
         _check(lib.dnpeff_csr_head_info(self._h, C.byref(nd), C.byref(zs)))
         return nd.value, zs.value
+
+    def products_info(self):
+        """dict(panels, plain, swept_pieces, tail_floor, list_entries, list_batches) of the sparse part."""
+        out = np.zeros(6, dtype=np.int64)
+        _check(lib.dnpeff_csr_products_info(self._h, _ptr(out)))
+        return dict(zip(("panels", "plain", "swept_pieces", "tail_floor", "list_entries", "list_batches"),
+                        (int(v) for v in out)))
 
     def build_transpose(self):
         _check(lib.dnpeff_csr_build_transpose(self._h))

@@ -165,10 +165,11 @@ struct tuning_t {
   double h_tile_mb = 768.0;        // size of a column tile of the tiled H update, MiB of the factor
   double tiled_h = -1.0;           // tiled H update: 1 = always, 0 = never, -1 = when the full-size buffer does not fit
   double topk_fast_cap = -1.0;     // top-k: candidate list length that ends the histogram passes (-1 = default)
-  double n_lists = 0.0;            // A H^T from slot lists on component slices (1 = on)
+  double n_lists = -1.0;           // A H^T from slot lists on component slices: 0 = never, 1 = the whole sparse
+                                   // part, 2 = its far tail, -1 = the far tail where that pays (see use_nlists_tail)
   double t_lists = 0.0;            // A^T W in column blocks on component slices (1 = on)
-  double nl_piece_cols = 16384.0;  // columns per piece of the slot lists
-  double nl_lag = 1.0;             // pieces the workgroups of an XCD may be apart
+  double nl_piece_cols = 32768.0;  // columns per piece of the slot lists
+  double nl_lag = 0.0;             // pieces the workgroups of an XCD may be apart
   double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
   double gram_fold = 1.0;          // diagonal tiles of X^T X with the work their symmetry leaves (0 = all sixteen blocks)
   double nl_wgs = 64.0;            // workgroups of the slot-list kernel per XCD (two per CU)
@@ -203,8 +204,10 @@ struct panel_plan {
   int coarse = 0;
   int sweep_cols = 0;
   double sweep_min = 0.0;
+  bool tail_lists = false;  // the plain panels past the last swept one go to slot lists instead
   bool operator==(const panel_plan& o) const {
-    return coarse == o.coarse && sweep_cols == o.sweep_cols && sweep_min == o.sweep_min;
+    return coarse == o.coarse && sweep_cols == o.sweep_cols && sweep_min == o.sweep_min &&
+           tail_lists == o.tail_lists;
   }
 };
 
@@ -212,7 +215,8 @@ struct panel_plan {
 // stream of (local row, local column, value) per wave slot, ordered by column piece.
 struct slot_lists {
   int piece_cols = 0, n_pieces = 0, n_parts = 0, rpw = 0, wgs = 0;
-  int64_t n_batches = 0;
+  int32_t floor_col = 0;          // the lists hold the entries of columns floor_col .. only
+  int64_t n_batches = 0, n_entries = 0;
   uint2* pairs = nullptr;         // [n_batches + 8][64]
   int64_t* slot_base = nullptr;   // [n_slots + 1] first batch of each slot
   uint32_t* off = nullptr;        // [n_slots][n_pieces + 1] batches of the slot before piece p
@@ -277,6 +281,10 @@ struct dnpeff_csr {
   int64_t* seg = nullptr;
   int32_t* pcol = nullptr;
   float* pval = nullptr;
+  // tail_floor > 0: the panels hold the entries of columns below tail_floor only (row i's at
+  // prow[i] .. prow[i + 1] of pcol / pval), the others are in the slot lists nl
+  int32_t tail_floor = 0;
+  int64_t* prow = nullptr;
   // after dnpeff_csr_split_dense_head: the dense block and the matrix of the remaining entries
   // (same shape, owned), which carries the derived structures the products use
   dn::slot_lists nl;
@@ -298,8 +306,9 @@ int csr_ensure_partials(dnpeff_csr* A, int r);
 int csr_set_panels(dnpeff_csr* S, const panel_plan& plan);
 // Swept panels are summed per XCD: one slot of partial sums per plain panel plus SWEEP_XCDS.
 constexpr int SWEEP_XCDS = 8;
+// With a far tail on slot lists (tail_floor > 0) their sums take one more slot, the last.
 inline int64_t panel_slots(const dnpeff_csr* S) {
-  return S->n_plain + (S->n_swept > 0 ? SWEEP_XCDS : 0);
+  return S->n_plain + (S->n_swept > 0 ? SWEEP_XCDS : 0) + (S->tail_floor > 0 ? 1 : 0);
 }
 // Whether the workgroups of a launch go to the SWEEP_XCDS XCDs round-robin (probed once).
 bool xcd_round_robin();
@@ -337,16 +346,22 @@ inline bool has_row_major(const dnpeff_csr* A) {
 }
 // lists.hip
 bool nlists_supported(const dnpeff_csr* S, int r);
-int nlists_build(dnpeff_csr* S, int r);
+// max_extra_bytes >= 0: the lists are not built (*declined = true) when they would take more than
+// that beyond the 8 bytes per entry of the panel copy they replace
+int nlists_build(dnpeff_csr* S, int r, int32_t floor_col = 0, double max_extra_bytes = -1.0,
+                 bool* declined = nullptr);
+int nlists_slots(int64_t n_rows, int r);  // wave slots (of eight lane groups) the lists of rank r use
+int csr_rows_count_below(const dnpeff_csr* S, int32_t col, int* d_below);
 void nlists_drop(dnpeff_csr* S);
-int launch_spmm_n_lists(const dnpeff_csr* S, int r, const float* H_mr, float* part);
+int launch_spmm_n_lists(const dnpeff_csr* S, int r, const float* H_mr, float* part, int64_t stride);
 int nlists_get_row(const dnpeff_csr* S, int64_t row, std::vector<int32_t>& cols, std::vector<float>& vals);
 bool tlists_supported(const dnpeff_csr* S, int r);
 int tblocks_build(dnpeff_csr* S);
 void tblocks_drop(dnpeff_csr* S);
 int launch_spmm_t_lists(const dnpeff_csr* S, int r, const float* W_nr, float* T, int64_t col0, int64_t col1);
 // Whether the products of the sparse part S at rank r run from the slot lists / column blocks.
-bool use_nlists(const dnpeff_csr* S, int r);
+bool use_nlists(const dnpeff_csr* S, int r);       // the whole sparse part on slot lists
+bool use_nlists_tail(const dnpeff_csr* S, int r);  // its far tail only
 bool use_tlists(const dnpeff_csr* S, int r);
 struct head_choice {
   int64_t thr = 0;   // columns with at least thr entries form the head (0 = no head)

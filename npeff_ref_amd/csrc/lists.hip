@@ -75,8 +75,8 @@ __global__ void __launch_bounds__(64 * NL_WAVES, 4)
     k_spmm_n_lists(const uint2* __restrict__ pairs, const int64_t* __restrict__ slot_base,
                    const uint32_t* __restrict__ off, int n_pieces, int piece_cols,
                    const int32_t* __restrict__ slot_rows, int rpw, int unit0, int n_units, int n_slices,
-                   int r, const float* __restrict__ H, float* __restrict__ N, int* __restrict__ progress,
-                   int lag, int spin_max) {
+                   int r, const float* __restrict__ H, float* __restrict__ N, int64_t n_stride,
+                   int* __restrict__ progress, int lag, int spin_max) {
   extern __shared__ __align__(16) float nl_sums[];  // [NL_WAVES][rpw][32]
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int x = blockIdx.x % SWEEP_XCDS, q = blockIdx.x / SWEEP_XCDS;
@@ -204,7 +204,7 @@ __global__ void __launch_bounds__(64 * NL_WAVES, 4)
   const int c = lane & 31;
   for (int lr = lane >> 5; lr < rpw; lr += 2) {
     const int row = slot_rows[(size_t)slot * rpw + lr];
-    if (row >= 0) N[(int64_t)row * r + slice * NL_SLICE + c] = my[lr * NL_SLICE + c];
+    if (row >= 0) N[(int64_t)row * n_stride + slice * NL_SLICE + c] = my[lr * NL_SLICE + c];
   }
 }
 
@@ -354,15 +354,18 @@ __global__ void __launch_bounds__(256)
 // ---------------------------------------------------------------------------
 // cnt[row][p] = entries of the row in piece p (one wave per row)
 __global__ void __launch_bounds__(64)
-    k_nl_row_count(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind, int n_pieces,
-                   int piece_cols, uint32_t* __restrict__ cnt) {
+    k_nl_row_count(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind, int32_t floor_col,
+                   int n_pieces, int piece_cols, uint32_t* __restrict__ cnt) {
   extern __shared__ int nl_lds[];
   const int64_t row = blockIdx.x;
   const int lane = threadIdx.x;
   for (int p = lane; p < n_pieces; p += 64) nl_lds[p] = 0;
   __syncthreads();
   const int64_t e1 = rowptr[row + 1];
-  for (int64_t e = rowptr[row] + lane; e < e1; e += 64) atomicAdd(&nl_lds[colind[e] / piece_cols], 1);
+  for (int64_t e = rowptr[row] + lane; e < e1; e += 64) {
+    const int col = colind[e] - floor_col;  // (entries below the floor are not the lists')
+    if (col >= 0) atomicAdd(&nl_lds[col / piece_cols], 1);
+  }
   __syncthreads();
   for (int p = lane; p < n_pieces; p += 64) cnt[row * n_pieces + p] = (uint32_t)nl_lds[p];
 }
@@ -430,7 +433,7 @@ __device__ inline int64_t nl_place(const int64_t* __restrict__ slot_base, const 
 // batch of 64 entries the rank among the entries of the same piece comes from ballots over the
 // bits of the piece number.
 __global__ void __launch_bounds__(64)
-    k_nl_scatter(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
+    k_nl_scatter(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind, int32_t floor_col,
                  const float* __restrict__ vals, const int32_t* __restrict__ row_slot,
                  const int32_t* __restrict__ slot_rows, int rpw, const uint32_t* __restrict__ cnt,
                  int n_pieces, int piece_cols, int piece_bits, const int64_t* __restrict__ slot_base,
@@ -451,11 +454,12 @@ __global__ void __launch_bounds__(64)
   const int64_t e0 = rowptr[row], e1 = rowptr[row + 1];
   for (int64_t base = e0; base < e1; base += 64) {
     const int64_t e = base + lane;
-    const bool active = e < e1;
+    bool active = e < e1;
     int p = 0, lcol = 0;
     float v = 0.0f;
+    const int col = active ? colind[e] - floor_col : -1;
+    active = col >= 0;
     if (active) {
-      const int col = colind[e];
       v = vals[e];
       p = col / piece_cols;
       lcol = col - p * piece_cols;
@@ -527,6 +531,8 @@ static int nlists_parts(int64_t n_rows, int r) {
   return parts < 1 ? 1 : parts;
 }
 
+int nlists_slots(int64_t n_rows, int r) { return nlists_parts(n_rows, r) * nlists_wgs() * NL_WAVES; }
+
 bool nlists_supported(const dnpeff_csr* S, int r) {
   if (r < NL_SLICE || r % NL_SLICE != 0 || r > 1024) return false;
   if (S->n_rows < 1 || S->n_rows >= ((int64_t)1 << 24) || S->nnz < 1) return false;
@@ -534,21 +540,50 @@ bool nlists_supported(const dnpeff_csr* S, int r) {
   return (int64_t)nlists_parts(S->n_rows, r) * nlists_wgs() * NL_WAVES <= NL_MAX_SLOTS;
 }
 
-int nlists_build(dnpeff_csr* S, int r) {
+// below[row] = entries of the row in columns < col (a row holds its entries in any order); one
+// wave per row
+__global__ void __launch_bounds__(256)
+    k_rows_count_below(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind, int64_t n_rows,
+                       int32_t col, int* __restrict__ below) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t e1 = rowptr[row + 1];
+  int c = 0;
+  for (int64_t e = rowptr[row] + lane; e < e1; e += 64) c += colind[e] < col;
+  for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+  if (lane == 0) below[row] = c;
+}
+
+int csr_rows_count_below(const dnpeff_csr* S, int32_t col, int* d_below) {
+  DN_CHECK(has_row_major(S), "row-major copy of the matrix was released");
+  if (S->n_rows == 0) return 0;
+  hipLaunchKernelGGL(k_rows_count_below, dim3((unsigned)ceil_div(S->n_rows, 4)), dim3(256), 0, stream(),
+                     S->rowptr, S->colind, S->n_rows, col, d_below);
+  DN_LAUNCH_CHECK();
+  return 0;
+}
+
+// floor_col > 0: lists of the entries in columns floor_col .. only (the far tail; the columns
+// below stay with the panels and swept pieces), columns counted from floor_col.
+int nlists_build(dnpeff_csr* S, int r, int32_t floor_col, double max_extra_bytes, bool* declined) {
+  if (declined) *declined = false;
   const tuning_t& tn = tuning();
   int piece_cols = (int)tn.nl_piece_cols;
   if (piece_cols < 64) piece_cols = 64;
-  if (piece_cols > 32768) piece_cols = 32768;
-  while (piece_cols < 32768 && ceil_div(S->n_cols, piece_cols) > NL_MAX_PIECES) piece_cols += 1024;
+  if (piece_cols > 65536) piece_cols = 65536;
+  while (piece_cols < 65536 && ceil_div(S->n_cols - floor_col, piece_cols) > NL_MAX_PIECES) piece_cols += 1024;
   const int n_parts = nlists_parts(S->n_rows, r);
   slot_lists& L = S->nl;
   const int wgs = nlists_wgs();
-  if (L.pairs && L.piece_cols == piece_cols && L.n_parts == n_parts && L.wgs == wgs) return 0;
+  if (L.pairs && L.piece_cols == piece_cols && L.n_parts == n_parts && L.wgs == wgs && L.floor_col == floor_col)
+    return 0;
   nlists_drop(S);
   DN_CHECK(nlists_supported(S, r), "no slot lists for %lld rows at rank %d", (long long)S->n_rows, r);
   DN_CHECK(has_row_major(S), "slot lists are built from the row-major copy, which was released");
   hipStream_t st = stream();
-  const int64_t n = S->n_rows, m = S->n_cols, z = S->nnz;
+  DN_CHECK(floor_col >= 0 && floor_col < S->n_cols, "slot lists: column floor %d", (int)floor_col);
+  const int64_t n = S->n_rows, m = S->n_cols - floor_col;
   const int n_slots = n_parts * wgs * NL_WAVES;
   const int rpw = 8 * (int)ceil_div(n, (int64_t)n_slots * 8);
   DN_CHECK(rpw <= NL_RPW_MAX, "slot lists: %d rows per slot", rpw);
@@ -558,13 +593,26 @@ int nlists_build(dnpeff_csr* S, int r) {
   // rows to (slot, lane group): longest first, dealt back and forth over the 8 n_slots groups, so
   // that the groups hold about the same number of entries (all slots of an XCD advance piece by
   // piece together, and a wave's eight groups step by step); local row = 8 * round + group
-  std::vector<int64_t> rowptr((size_t)n + 1);
+  std::vector<int64_t> rowptr((size_t)n + 1), mine((size_t)n);  // mine: the row's entries in the lists
+  std::vector<int> below((size_t)n, 0);
+  if (floor_col > 0) {
+    dbuf<int> d_below;
+    DN_TRY(d_below.alloc(n));
+    DN_TRY(csr_rows_count_below(S, floor_col, d_below.p));
+    DN_HIP(hipStreamSynchronize(st));
+    DN_HIP(hipMemcpy(below.data(), d_below.p, sizeof(int) * n, hipMemcpyDeviceToHost));
+  }
   DN_HIP(hipStreamSynchronize(st));
   DN_HIP(hipMemcpy(rowptr.data(), S->rowptr, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToHost));
+  int64_t z = 0;
+  for (int64_t i = 0; i < n; i++) {
+    mine[(size_t)i] = rowptr[(size_t)i + 1] - rowptr[(size_t)i] - below[(size_t)i];
+    z += mine[(size_t)i];
+  }
   std::vector<int32_t> order((size_t)n), row_slot((size_t)n), slot_rows((size_t)n_slots * rpw, -1);
   for (int64_t i = 0; i < n; i++) order[(size_t)i] = (int32_t)i;
   std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) {
-    return rowptr[(size_t)a + 1] - rowptr[(size_t)a] > rowptr[(size_t)b + 1] - rowptr[(size_t)b];
+    return mine[(size_t)a] > mine[(size_t)b];
   });
   const int64_t n_groups = (int64_t)n_slots * 8;
   for (int64_t t = 0; t < n; t++) {
@@ -586,8 +634,8 @@ int nlists_build(dnpeff_csr* S, int r) {
   DN_HIP(hipMemcpy(L.row_slot, row_slot.data(), sizeof(int32_t) * n, hipMemcpyHostToDevice));
   DN_HIP(hipMemcpy(L.slot_rows, slot_rows.data(), sizeof(int32_t) * slot_rows.size(), hipMemcpyHostToDevice));
   const size_t lds = sizeof(int) * (size_t)n_pieces;
-  hipLaunchKernelGGL(k_nl_row_count, dim3((unsigned)n), dim3(64), lds, st, S->rowptr, S->colind, n_pieces,
-                     piece_cols, cnt.p);
+  hipLaunchKernelGGL(k_nl_row_count, dim3((unsigned)n), dim3(64), lds, st, S->rowptr, S->colind, floor_col,
+                     n_pieces, piece_cols, cnt.p);
   DN_LAUNCH_CHECK();
   hipLaunchKernelGGL(k_nl_slot_batches, dim3((unsigned)ceil_div((int64_t)n_slots * n_pieces, 256)), dim3(256), 0,
                      st, cnt.p, L.slot_rows, rpw, n_pieces, n_slots, nbat.p);
@@ -605,13 +653,21 @@ int nlists_build(dnpeff_csr* S, int r) {
   const int64_t n_batches = L.h_slot_base[(size_t)n_slots];
   DN_HIP(hipMemcpy(L.slot_base, L.h_slot_base.data(), sizeof(int64_t) * ((size_t)n_slots + 1),
                    hipMemcpyHostToDevice));
+  if (max_extra_bytes >= 0.0 && (double)(n_batches + 8) * 512.0 - 8.0 * (double)z > max_extra_bytes) {
+    if (tn.verbose != 0.0)
+      fprintf(stderr, "dnpeff: slot lists of %lld entries would take %.2f GB: not built\n", (long long)z,
+              (double)(n_batches + 8) * 512.0 / 1e9);
+    nlists_drop(S);
+    if (declined) *declined = true;
+    return 0;
+  }
   // (the kernel requests pairs up to seven batches past a slot's last)
   DN_TRY(dmalloc(&L.pairs, (n_batches + 8) * 64));
   DN_HIP(hipMemsetAsync(L.pairs + n_batches * 64, 0, sizeof(uint2) * 8 * 64, st));
   int piece_bits = 0;
   while ((1 << piece_bits) < n_pieces) piece_bits++;
-  hipLaunchKernelGGL(k_nl_scatter, dim3((unsigned)n), dim3(64), lds, st, S->rowptr, S->colind, S->vals,
-                     L.row_slot, L.slot_rows, rpw, cnt.p, n_pieces, piece_cols, piece_bits, L.slot_base, L.off,
+  hipLaunchKernelGGL(k_nl_scatter, dim3((unsigned)n), dim3(64), lds, st, S->rowptr, S->colind, floor_col,
+                     S->vals, L.row_slot, L.slot_rows, rpw, cnt.p, n_pieces, piece_cols, piece_bits, L.slot_base, L.off,
                      L.pairs);
   DN_LAUNCH_CHECK();
   hipLaunchKernelGGL(k_nl_fill, dim3((unsigned)ceil_div((int64_t)n_slots * n_pieces * 8, 256)), dim3(256), 0, st,
@@ -619,6 +675,8 @@ int nlists_build(dnpeff_csr* S, int r) {
   DN_LAUNCH_CHECK();
   DN_HIP(hipStreamSynchronize(st));
   L.piece_cols = piece_cols;
+  L.floor_col = floor_col;
+  L.n_entries = z;
   L.n_pieces = n_pieces;
   L.n_parts = n_parts;
   L.wgs = wgs;
@@ -627,9 +685,9 @@ int nlists_build(dnpeff_csr* S, int r) {
   L.h_row_slot = std::move(row_slot);
   if (tn.verbose != 0.0)
     fprintf(stderr,
-            "dnpeff: slot lists: %d part(s) x %d slots of %d rows, %d pieces of %d columns, %lld batches "
-            "(%.1f %% filler), %.2f GB\n",
-            n_parts, wgs * NL_WAVES, rpw, n_pieces, piece_cols, (long long)n_batches,
+            "dnpeff: slot lists of %lld entries from column %d on: %d part(s) x %d slots of %d rows, %d pieces of "
+            "%d columns, %lld batches (%.1f %% filler), %.2f GB\n",
+            (long long)z, (int)floor_col, n_parts, wgs * NL_WAVES, rpw, n_pieces, piece_cols, (long long)n_batches,
             z > 0 ? 100.0 * ((double)n_batches * 64.0 / (double)z - 1.0) : 0.0,
             (double)(n_batches + 8) * 512.0 / 1e9);
   return 0;
@@ -637,11 +695,11 @@ int nlists_build(dnpeff_csr* S, int r) {
 
 __global__ void k_nl_clear(int* progress) { progress[threadIdx.x] = 0; }
 
-// part[row, :] = the sparse part's share of (A H^T)[row, :]
-int launch_spmm_n_lists(const dnpeff_csr* S, int r, const float* H_mr, float* part) {
+// part[row * stride .. + r) = the listed entries' share of (A H^T)[row, :] (stride in floats)
+int launch_spmm_n_lists(const dnpeff_csr* S, int r, const float* H_mr, float* part, int64_t stride) {
   const slot_lists& L = S->nl;
   DN_CHECK(L.pairs != nullptr, "matrix has no slot lists");
-  DN_CHECK(r % NL_SLICE == 0 && ((uintptr_t)H_mr % 16) == 0, "slot lists: rank %d or alignment", r);
+  DN_CHECK(r % NL_SLICE == 0 && ((uintptr_t)H_mr % 16) == 0 && stride >= r, "slot lists: rank %d or alignment", r);
   DN_CHECK(L.n_parts == nlists_parts(S->n_rows, r) && L.wgs == nlists_wgs(), "slot lists were built for another rank");
   static bool attr_set = false;
   const size_t lds = (size_t)NL_WAVES * L.rpw * NL_ROW_BYTES;
@@ -658,7 +716,7 @@ int launch_spmm_n_lists(const dnpeff_csr* S, int r, const float* H_mr, float* pa
     hipLaunchKernelGGL(k_nl_clear, dim3(1), dim3(SWEEP_XCDS * NL_SYNC_STRIDE), 0, stream(), L.progress);
     hipLaunchKernelGGL(k_spmm_n_lists, dim3(SWEEP_XCDS * L.wgs), dim3(64 * NL_WAVES), lds, stream(), L.pairs,
                        L.slot_base, L.off, L.n_pieces, L.piece_cols, L.slot_rows, L.rpw, unit0, n_units,
-                       n_slices, r, H_mr, part, L.progress, lag, spin_max);
+                       n_slices, r, H_mr + (int64_t)L.floor_col * r, part, stride, L.progress, lag, spin_max);
     DN_LAUNCH_CHECK();
     if (tn.verbose >= 2.0) {  // how the lock step went: counts past NL_GIVE_UP mean a wait ran out
       int h[SWEEP_XCDS * NL_SYNC_STRIDE];
@@ -695,7 +753,7 @@ int nlists_get_row(const dnpeff_csr* S, int64_t row, std::vector<int32_t>& cols,
       for (int k = 0; k < 8; k++) {
         const uint2 e = pairs[b * 64 + (size_t)g * 8 + k];
         if ((int)(e.x >> 16) == lrow * NL_ROW_BYTES && !((e.x & 0xffffu) == 0u && e.y == 0u)) {
-          cols.push_back((int32_t)((int64_t)p * L.piece_cols + (e.x & 0xffffu)));
+          cols.push_back((int32_t)(L.floor_col + (int64_t)p * L.piece_cols + (e.x & 0xffffu)));
           float v;
           memcpy(&v, &e.y, sizeof(float));
           vals.push_back(v);

@@ -309,7 +309,12 @@ __global__ void __launch_bounds__(256)
     k_panel_split(const int64_t* __restrict__ rowptr, const int32_t* __restrict__ colind,
                   const float* __restrict__ vals, int64_t n_rows, int P, int bits,
                   const int32_t* __restrict__ bounds, int64_t* __restrict__ seg,
-                  int32_t* __restrict__ pcol, float* __restrict__ pval) {
+                  int32_t* __restrict__ pcol, float* __restrict__ pval,
+                  const int64_t* __restrict__ out_begin) {
+  // out_begin (or NULL): the panels end below the matrix's last column; row i's entries below
+  // bounds[P] (out_begin[i + 1] - out_begin[i] of them, anywhere in the row) go to
+  // out_begin[i] .. of pcol / pval, and the segment offsets count from there; the others are left
+  // out
   __shared__ int32_t bnd[MAX_PANELS + 1];
   __shared__ int hist[MAX_PANELS];
   __shared__ int cursor[MAX_PANELS];         // next free position of each panel, relative to e0
@@ -326,13 +331,17 @@ __global__ void __launch_bounds__(256)
   };
   for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
     const int64_t e0 = rowptr[row], e1 = rowptr[row + 1];
+    const int64_t o0 = out_begin ? out_begin[row] : e0;
+    const int64_t o1 = out_begin ? out_begin[row + 1] : e1;
+    const int32_t col_end = bounds[P];
     __syncthreads();
     for (int i = tid; i < P; i += 256) {
       hist[i] = 0;
       wcnt[0][i] = wcnt[1][i] = wcnt[2][i] = wcnt[3][i] = 0;
     }
     __syncthreads();
-    for (int64_t e = e0 + tid; e < e1; e += 256) atomicAdd(&hist[panel_of(colind[e])], 1);
+    for (int64_t e = e0 + tid; e < e1; e += 256)
+      if (colind[e] < col_end) atomicAdd(&hist[panel_of(colind[e])], 1);
     __syncthreads();
     // exclusive scan of the panel counts: each thread sums a run of consecutive panels, the
     // run totals are scanned by thread 0
@@ -356,21 +365,24 @@ __global__ void __launch_bounds__(256)
         int run = cursor[p0];
         for (int q = p0; q < p0 + per && q < P; q++) {
           cursor[q] = run;
-          seg[row * (P + 1) + q] = e0 + run;
+          seg[row * (P + 1) + q] = o0 + run;
           run += hist[q];
         }
       }
     }
-    if (tid == 0) seg[row * (P + 1) + P] = e1;
+    if (tid == 0) seg[row * (P + 1) + P] = o1;
     __syncthreads();
     for (int64_t base = e0; base < e1; base += 256) {
       const int64_t e = base + tid;
-      const bool active = e < e1;
+      bool active = e < e1;
       int32_t col = 0;
       float v = 0.0f;
       int pid = 0;
       if (active) {
         col = colind[e];
+        active = col < col_end;
+      }
+      if (active) {
         v = vals[e];
         pid = panel_of(col);
       }
@@ -390,7 +402,7 @@ __global__ void __launch_bounds__(256)
           if (w < wave) off += c;
           tot += c;
         }
-        const int64_t pos = e0 + cursor[pid] + off + rank;
+        const int64_t pos = o0 + cursor[pid] + off + rank;
         pcol[pos] = col;
         pval[pos] = v;
       }
@@ -609,6 +621,8 @@ static void drop_panels(dnpeff_csr* A) {
   dfree(A->seg); A->seg = nullptr;
   dfree(A->pcol); A->pcol = nullptr;
   dfree(A->pval); A->pval = nullptr;
+  dfree(A->prow); A->prow = nullptr;
+  A->tail_floor = 0;
   if (A->n_panels) {  // the partial sums were sized for the panels
     dfree(A->partials); A->partials = nullptr; A->partials_floats = 0;
   }
@@ -668,13 +682,27 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
   // (spmm.hip).  A raised threshold keeps the number of panels within bounds.
   std::vector<int32_t> bounds, ids, swept;
   double min_seg = plan.sweep_min;
+  int P_used = P0;  // coarse panels that stay panels
   for (;;) {
     bounds.clear(); ids.clear(); swept.clear();
     const double per_coarse = (double)S->nnz / P0 / (double)(S->n_rows > 0 ? S->n_rows : 1);
-    for (int c = 0; c < P0; c++) {
+    auto sweeps = [&](int c) {
       const int64_t w = (int64_t)coarse[c + 1] - coarse[c];
-      const bool sweep = plan.sweep_cols > 0 && w > plan.sweep_cols + plan.sweep_cols / 4 &&
-                         per_coarse * (double)plan.sweep_cols / (double)w >= min_seg;
+      return plan.sweep_cols > 0 && w > plan.sweep_cols + plan.sweep_cols / 4 &&
+             per_coarse * (double)plan.sweep_cols / (double)w >= min_seg;
+    };
+    // The far tail: the plain panels past the last swept one.  With tail_lists their entries go
+    // to slot lists and the panels end at the first of them.
+    P_used = P0;
+    if (plan.tail_lists) {
+      int last_swept = -1;
+      for (int c = 0; c < P0; c++)
+        if (sweeps(c)) last_swept = c;
+      if (last_swept >= 0 && last_swept + 1 < P0 && coarse[last_swept + 1] > 0) P_used = last_swept + 1;
+    }
+    for (int c = 0; c < P_used; c++) {
+      const int64_t w = (int64_t)coarse[c + 1] - coarse[c];
+      const bool sweep = sweeps(c);
       const int64_t parts = sweep ? ceil_div(w, plan.sweep_cols) : 1;
       for (int64_t q = 0; q < parts; q++) {
         (sweep ? swept : ids).push_back((int32_t)bounds.size());
@@ -684,8 +712,22 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
     if ((int64_t)bounds.size() <= MAX_PANELS) break;
     min_seg = min_seg > 0.0 ? min_seg * 1.5 : 1.0;
   }
-  bounds.push_back((int32_t)S->n_cols);
+  const int32_t tail_floor = P_used < P0 ? coarse[P_used] : 0;
+  bounds.push_back(tail_floor > 0 ? tail_floor : (int32_t)S->n_cols);
   const int P = (int)bounds.size() - 1;
+  // rows' places in the panel copy when it leaves the far tail out
+  int64_t nnz_panels = S->nnz;
+  if (tail_floor > 0) {
+    dbuf<int> below;
+    int s0 = below.alloc(S->n_rows) || dmalloc(&S->prow, S->n_rows + 1) ||
+             csr_rows_count_below(S, tail_floor, below.p) ||
+             scan_counts_i64(below.p, S->n_rows, S->prow);
+    if (!s0 && hipMemcpy(&nnz_panels, S->prow + S->n_rows, sizeof(int64_t), hipMemcpyDeviceToHost) != hipSuccess) {
+      set_error("building the column panels failed (row prefixes)");
+      s0 = 1;
+    }
+    if (s0) { drop_panels(S); return 1; }
+  }
   const int n_plain = (int)ids.size(), n_swept = (int)swept.size();
   ids.insert(ids.end(), swept.begin(), swept.end());
 
@@ -693,8 +735,8 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
   while ((1 << bits) < P) bits++;
   int s = dmalloc(&S->panel_bounds, (int64_t)P + 1) || dmalloc(&S->panel_ids, (int64_t)P) ||
           dmalloc(&S->sweep_progress, 256) ||
-          dmalloc(&S->seg, S->n_rows * (P + 1)) || dmalloc(&S->pcol, S->nnz + 64) ||
-          dmalloc(&S->pval, S->nnz + 64);  // (the sweep kernel reads 64 pairs at a time)
+          dmalloc(&S->seg, S->n_rows * (P + 1)) || dmalloc(&S->pcol, nnz_panels + 64) ||
+          dmalloc(&S->pval, nnz_panels + 64);  // (the sweep kernel reads 64 pairs at a time)
   if (!s) {
     hipError_t e = hipMemcpy(S->panel_bounds, bounds.data(), sizeof(int32_t) * bounds.size(),
                              hipMemcpyHostToDevice);
@@ -704,7 +746,7 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
       int64_t wgs = S->n_rows < 8192 ? S->n_rows : 8192;
       hipLaunchKernelGGL(k_panel_split, dim3((unsigned)(wgs < 1 ? 1 : wgs)), dim3(256), 0, st,
                          S->rowptr, S->colind, S->vals, S->n_rows, P, bits, S->panel_bounds, S->seg,
-                         S->pcol, S->pval);
+                         S->pcol, S->pval, (const int64_t*)S->prow);
       e = hipGetLastError();
       if (e == hipSuccess) e = hipStreamSynchronize(st);
     }
@@ -718,9 +760,15 @@ int csr_set_panels(dnpeff_csr* S, const panel_plan& plan) {
   S->n_plain = n_plain;
   S->n_swept = n_swept;
   S->plan = plan;
-  if (tuning().verbose != 0.0)
-    fprintf(stderr, "dnpeff: %d column panels: %d plain, %d cut into %d swept pieces\n", P0, n_plain,
-            P0 - n_plain, n_swept);
+  S->tail_floor = tail_floor;
+  if (tuning().verbose != 0.0) {
+    fprintf(stderr, "dnpeff: %d column panels: %d plain, %d cut into %d swept pieces", P_used, n_plain,
+            P_used - n_plain, n_swept);
+    if (tail_floor > 0)
+      fprintf(stderr, "; the %d panels from column %d on (%lld entries) go to slot lists", P0 - P_used,
+              (int)tail_floor, (long long)(S->nnz - nnz_panels));
+    fprintf(stderr, "\n");
+  }
   dfree(S->partials); S->partials = nullptr; S->partials_floats = 0;
   return 0;
 }
@@ -786,7 +834,20 @@ static panel_plan panel_policy(const dnpeff_csr* S, int r) {
 // pieces and 4-slice column kernel that the plan uses otherwise.  Needs a rank that is a multiple
 // of 32 and workgroups dealt to the XCDs round-robin.
 bool use_nlists(const dnpeff_csr* S, int r) {
-  return tuning().n_lists > 0.0 && nlists_supported(S, r) && xcd_round_robin();
+  return tuning().n_lists == 1.0 && nlists_supported(S, r) && xcd_round_robin();
+}
+// The far tail only (the plain panels past the last swept one) on slot lists, beside the panels
+// and swept pieces of the columns before it: n_lists = 2 wherever the lists can be built; left to
+// itself (n_lists < 0) where it was measured to pay: ranks from 256 (eight slices or more: one per
+// XCD, the entry streams read once per slice) and four rows or more per lane group (with fewer,
+// the groups' lists of a piece are short and uneven, and most of a batch is filler): 195 against
+// 221 ms for A H^T at 20,000 x 211M, r = 256, 397 against 462 ms at 40,000 ragged rows, r = 512,
+// but 20.6 against 19.6 ms at 10,000 rows, r = 128.
+bool use_nlists_tail(const dnpeff_csr* S, int r) {
+  const double sw = tuning().n_lists;
+  if (!(sw == 2.0 || sw < 0.0) || !nlists_supported(S, r) || !xcd_round_robin()) return false;
+  if (sw == 2.0) return true;
+  return r >= 256 && S->n_rows >= 4 * 8 * (int64_t)nlists_slots(S->n_rows, r);
 }
 bool use_tlists(const dnpeff_csr* S, int r) {
   return tuning().t_lists > 0.0 && tlists_supported(S, r) && xcd_round_robin();
@@ -799,8 +860,23 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
     DN_TRY(csr_set_panels(S, panel_plan()));
     DN_TRY(nlists_build(S, r));
   } else {
-    nlists_drop(S);
-    DN_TRY(csr_set_panels(S, panel_policy(S, r)));
+    panel_plan plan = panel_policy(S, r);
+    plan.tail_lists = plan.coarse > 0 && plan.sweep_cols > 0 && use_nlists_tail(S, r);
+    DN_TRY(csr_set_panels(S, plan));
+    if (S->tail_floor > 0) {
+      // Left to itself, the plan gives the lists what the panel copy of the same entries would
+      // take plus half of the memory that the plan keeps free; beyond that the tail stays panels.
+      size_t free_b = 0, total_b = 0;
+      DN_HIP(hipMemGetInfo(&free_b, &total_b));
+      bool declined = false;
+      DN_TRY(nlists_build(S, r, S->tail_floor, tuning().n_lists < 0.0 ? (double)total_b / 128.0 : -1.0, &declined));
+      if (declined) {
+        plan.tail_lists = false;
+        DN_TRY(csr_set_panels(S, plan));
+      }
+    } else {
+      nlists_drop(S);
+    }
   }
   if (use_tlists(S, r)) DN_TRY(tblocks_build(S));
   DN_TRY(csr_ensure_partials(S, r));
@@ -1415,6 +1491,18 @@ DN_API int dnpeff_csr_head_info(const dnpeff_csr* A, int64_t* n_dense, int64_t* 
   return 0;
 }
 
+DN_API int dnpeff_csr_products_info(const dnpeff_csr* A, int64_t* out6) {
+  DN_CHECK(A != nullptr && out6 != nullptr, "NULL argument");
+  const dnpeff_csr* S = sparse_part(A);
+  out6[0] = S->n_panels;
+  out6[1] = S->n_plain;
+  out6[2] = S->n_swept;
+  out6[3] = S->tail_floor;
+  out6[4] = S->nl.pairs ? S->nl.n_entries : 0;
+  out6[5] = S->nl.pairs ? S->nl.n_batches : 0;
+  return 0;
+}
+
 DN_API int dnpeff_csr_build_transpose(dnpeff_csr* A) {
   clear_error();
   DN_CHECK(A != nullptr, "matrix is NULL");
@@ -1541,14 +1629,30 @@ DN_API int dnpeff_csr_get_row(dnpeff_csr* A, int64_t row, int64_t cap, int64_t* 
   const float* src_v = S->vals ? S->vals : S->pval;
   std::vector<int32_t> list_cols;
   std::vector<float> list_vals;
-  if (!(src_c && src_v) && S->nl.pairs) {  // the sparse part is held as slot lists
+  const int64_t row_entries = e[1] - e[0];
+  if (!S->colind && S->pcol && S->tail_floor > 0 && S->nl.pairs) {
+    // the panels hold the row's entries below tail_floor, the slot lists the others
     DN_TRY(nlists_get_row(S, row, list_cols, list_vals));
-    DN_CHECK((int64_t)list_cols.size() == e[1] - e[0], "slot lists hold %lld entries of row %lld, not %lld",
-             (long long)list_cols.size(), (long long)row, (long long)(e[1] - e[0]));
+    DN_HIP(hipMemcpy(e, S->prow + row, sizeof(e), hipMemcpyDeviceToHost));
+    DN_CHECK((int64_t)list_cols.size() + (e[1] - e[0]) == row_entries,
+             "panels and slot lists hold %lld entries of row %lld, not %lld",
+             (long long)((int64_t)list_cols.size() + (e[1] - e[0])), (long long)row, (long long)row_entries);
+    std::vector<int32_t> pc((size_t)(e[1] - e[0]));
+    std::vector<float> pv((size_t)(e[1] - e[0]));
+    if (e[1] > e[0]) {
+      DN_HIP(hipMemcpy(pc.data(), S->pcol + e[0], sizeof(int32_t) * pc.size(), hipMemcpyDeviceToHost));
+      DN_HIP(hipMemcpy(pv.data(), S->pval + e[0], sizeof(float) * pv.size(), hipMemcpyDeviceToHost));
+    }
+    list_cols.insert(list_cols.begin(), pc.begin(), pc.end());
+    list_vals.insert(list_vals.begin(), pv.begin(), pv.end());
+  } else if (!(src_c && src_v) && S->nl.pairs) {  // the sparse part is held as slot lists
+    DN_TRY(nlists_get_row(S, row, list_cols, list_vals));
+    DN_CHECK((int64_t)list_cols.size() == row_entries, "slot lists hold %lld entries of row %lld, not %lld",
+             (long long)list_cols.size(), (long long)row, (long long)row_entries);
   } else {
     DN_CHECK(e[1] == e[0] || (src_c && src_v), "matrix holds no row-major copy of its sparse part");
   }
-  int64_t got = e[1] - e[0];
+  int64_t got = row_entries;
   std::vector<float> head_row;
   std::vector<int32_t> head_cols;
   if (A->head.n_d) {

@@ -1184,7 +1184,7 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
   float* partials = A->partials;
   if (A->nl.pairs && use_nlists(A, r)) {
     DN_CHECK(partials && A->partials_floats >= A->n_rows * (int64_t)r, "partial sums too small");
-    return launch_spmm_n_lists(A, r, H_mr, partials);
+    return launch_spmm_n_lists(A, r, H_mr, partials, r);
   }
   if (A->n_panels > 0) {
     DN_CHECK(A->seg && A->pcol && A->panel_ids && partials, "matrix has no panel work list");
@@ -1206,6 +1206,12 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
     if (A->n_swept > 0) {
       DN_TRY(side_stream_join());
       DN_TRY(launch_spmm_n_sweep(A, r, H_mr, aligned, slots));
+    }
+    // the far tail from its slot lists, into the last slot of the partial sums
+    if (A->tail_floor > 0) {
+      DN_CHECK(A->nl.pairs && A->nl.floor_col == A->tail_floor, "the far tail has no slot lists");
+      DN_TRY(side_stream_join());
+      DN_TRY(launch_spmm_n_lists(A, r, H_mr, partials + (int64_t)(slots - 1) * r, (int64_t)slots * r));
     }
     return 0;
   }

@@ -25,7 +25,7 @@ pytestmark = pytest.mark.gpu
 TOL = 2e-5
 
 
-def _full_size_checks(n, m_full, k, zipf_s, r, seed, n_rows_sampled, tiled_expected, k_min=0, k_max=0):
+def _full_size_checks(n, m_full, k, zipf_s, r, seed, n_rows_sampled, tiled_expected, k_min=0, k_max=0, tail_lists_expected=False):
     A, norms = d.Csr.synth(n, m_full, k_fixed=k, k_min=k_min, k_max=k_max, zipf_s=zipf_s, seed=seed)
     A.normalize_rows(norms)
     A.compact_columns(1)
@@ -72,6 +72,9 @@ def _full_size_checks(n, m_full, k, zipf_s, r, seed, n_rows_sampled, tiled_expec
     d.binding._check(d.lib.dnpeff_op_spmm_n(A._h, r, C.c_void_p(h_dev), N_dev.ptr))
     d.sync()
     N = N_dev.numpy()
+    # how the sparse part ran: at ranks from 256 with rows enough, the far tail from slot lists
+    info = A.products_info()
+    assert (info["tail_floor"] > 0 and info["list_entries"] > 0) == tail_lists_expected, info
 
     rng = np.random.default_rng(seed % 1000)
     rows = np.unique(np.concatenate([[0, n // 3, n - 1], rng.integers(0, n, n_rows_sampled)]))[:n_rows_sampled]
@@ -132,7 +135,7 @@ def test_configs3_at_full_size():
     if total < 280e9:
         pytest.skip("configs[3] needs the 288 GB of an MI355X")
     _full_size_checks(20_000, 350_000_000, 262_144, 1.3, 256, 43190432042, n_rows_sampled=8,
-                      tiled_expected=True)
+                      tiled_expected=True, tail_lists_expected=True)
 
 
 @pytest.mark.timeout(600)
@@ -142,7 +145,7 @@ def test_configs4_ragged_rows_at_full_size():
     if total < 280e9:
         pytest.skip("configs[4] needs the 288 GB of an MI355X")
     _full_size_checks(40_000, 110_000_000, 0, 1.1, 512, 43190432042, n_rows_sampled=6, tiled_expected=True,
-                      k_min=1_024, k_max=524_288)
+                      k_min=1_024, k_max=524_288, tail_lists_expected=True)
 
 
 def test_configs2_fit_path_at_full_size():

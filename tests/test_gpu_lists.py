@@ -130,3 +130,80 @@ def test_nmf_on_slices_matches_oracle_and_inspection_after_consume(r, n, tune):
     assert np.array_equal(nmf.loadWToHostSync(), W) and np.array_equal(nmf.loadHToHostSync(), H)
     nmf.close()
     A.close()
+
+
+def _tail_plan(tune, r, piece_cols=2000, sweep_min=50):
+    """Six coarse panels of which the widest (the last) holds too few entries per row and piece to
+    be swept: with n_lists = 2 its entries go to slot lists, the others stay panels and pieces."""
+    tune("n_lists", 2)
+    tune("panels", 6)
+    tune("sweep_bytes", piece_cols * 4 * min(r, 256))  # (ranks above 256 are swept in slices of 256)
+    tune("sweep_min", sweep_min)
+    tune("nl_piece_cols", 1024)
+
+
+@pytest.mark.parametrize("r", [64, 128, 256, 512])
+def test_far_tail_from_slot_lists_beside_panels_and_pieces(r, tune):
+    _tail_plan(tune, r)
+    rng = np.random.default_rng(r)
+    n, m_full = 300, 40000
+    rowptr, colind, vals, _ = d.synth_pef_host(n, m_full, k_fixed=2048, zipf_s=1.1, seed=9)
+    A = d.Csr.from_host(rowptr, colind, vals, m_full)
+    H = rng.random((m_full, r)).astype(np.float32)
+    dH, dN = d.DeviceArray.from_numpy(H), d.DeviceArray((n, r))
+    d.op_spmm_n(A, r, dH, dN)
+    info = A.products_info()
+    assert info["tail_floor"] > 0 and info["swept_pieces"] > 0
+    want_tail = int((colind >= info["tail_floor"]).sum())
+    assert info["list_entries"] == want_tail and 0 < want_tail < len(colind)
+    N = dN.numpy()
+    assert _row_rel(N.astype(np.float64), orc.spmm_n_f64(rowptr, colind, vals, H)) < TOL
+    d.op_spmm_n(A, r, dH, dN)
+    assert np.array_equal(dN.numpy(), N)
+    # the same product without the lists: same sums up to the order of the tail's entries
+    tune("n_lists", 0)
+    d.op_spmm_n(A, r, dH, dN)
+    assert A.products_info()["tail_floor"] == 0
+    assert _row_rel(dN.numpy().astype(np.float64), N.astype(np.float64)) < TOL
+    A.close()
+
+
+def test_nmf_with_the_far_tail_on_slot_lists(tune):
+    """A factorisation (dense head, consumed matrix) whose far tail runs from slot lists: 20
+    iterations against the fp64 oracle, rows read back from panels + lists, same bits again."""
+    r, n = 256, 2100
+    tune("n_lists", 2)
+    tune("panels", 8)
+    tune("sweep_bytes", 3000 * 4 * r)
+    tune("sweep_min", 40)
+    tune("nl_piece_cols", 2048)
+    m_full, k, iters, eps, seed = 100000, 2000, 20, 1e-12, 78
+    A, norms = d.Csr.synth(n, m_full, k_fixed=k, zipf_s=1.3, seed=seed)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    rp, ci, va = A.download()
+    m = A.n_cols
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=iters, eps=eps, seed=seed, log_every=10), consume_matrix=True)
+    info = A.products_info()
+    assert info["tail_floor"] > 0 and info["list_entries"] > 0 and info["swept_pieces"] > 0, info
+    for i in (0, 7, n // 2, n - 1):
+        cols, vals = A.get_row(i)
+        o = np.argsort(cols, kind="stable")
+        want_c, want_v = ci[rp[i]:rp[i + 1]], va[rp[i]:rp[i + 1]]
+        ow = np.argsort(want_c, kind="stable")
+        assert np.array_equal(cols[o], want_c[ow]) and np.array_equal(vals[o], want_v[ow])
+    nmf.initialize()
+    W0, H0 = nmf.loadWToHostSync(), nmf.loadHToHostSync()
+    hist = nmf.run(log=lambda s: None)
+    W, H = nmf.loadWToHostSync(), nmf.loadHToHostSync()
+    W64, H64, losses = orc.nmf_f64(rp, ci, va, m, W0, H0, np.float32(eps), iters, 10)
+    assert np.linalg.norm(W - W64) / np.linalg.norm(W64) < 1e-4
+    assert np.linalg.norm(H - H64) / np.linalg.norm(H64) < 1e-4
+    assert abs(hist[-1][1] - losses[-1]) / losses[-1] < 1e-4
+    via_rows, via_cols = nmf.check_products()
+    assert abs(via_rows - via_cols) <= 5e-6 * abs(via_rows)
+    nmf.initialize()
+    nmf.run(log=lambda s: None)
+    assert np.array_equal(nmf.loadWToHostSync(), W) and np.array_equal(nmf.loadHToHostSync(), H)
+    nmf.close()
+    A.close()
