@@ -9,8 +9,12 @@
 //   A H^T  (k_spmm_n_lists): XCD x sums components [32 x, 32 x + 32) of every row of the result.
 //     The running sums of all rows live in the LDS of the XCD's CUs (a wave slot owns up to 72
 //     rows, 512 slots per XCD), and all slots walk the columns in the same order, piece by piece
-//     (a piece: 16,384 columns, 2 MB of 128-byte row slices of H), so that a row slice of H is
-//     fetched from HBM once and found in the L2 by the other rows that use it.  The entries are
+//     (a piece: 32,768 columns, 4 MB of 128-byte row slices of H), so that a row slice of H is
+//     fetched from HBM once and found in the L2 by the other rows that use it.  This is how the
+//     far tail of a sparse part runs (the columns past the last swept piece, a few entries each,
+//     which as panels bring every gathered row over the fabric: lists from a column floor on,
+//     their sums in a slot of their own beside the panels' and the swept pieces'); the whole
+//     sparse part can run this way too (n_lists = 1) and is slower than panels and pieces then.  The entries are
 //     kept as one stream of (local row, local column, value) per slot, ordered by piece
 //     ("slot lists").  Each of the 8 lane groups of a wave owns every eighth row of the slot
 //     for good: it gathers one 128-byte slice per entry, sums the entries of a row in registers
