@@ -81,7 +81,8 @@ int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int
  * tiles of X^T X without the use of their symmetry), n_lists (A H^T from slot lists on component slices of 32: -1 =
  * the far tail of the sparse part where that was measured to pay, 2 = wherever possible, 1 = the
  * whole sparse part, 0 = never), t_lists (1: A^T W in column blocks on such slices), nl_piece_cols,
- * nl_lag, nl_spin, nl_wgs (their piece size, lock step and launch shape).
+ * nl_lag, nl_spin, nl_wgs (their piece size, lock step and launch shape), nl_extra_mb (memory the
+ * far tail's lists may take beyond the panel copy they replace).
  * Each starts from the environment variable DNPEFF_<NAME IN CAPITALS> (read once, when the
  * library is first used) or its default; plans take the values when they are made
  * (dnpeff_nmf_create, the first product on a matrix).  dnpeff_tuning_reset() goes back to the

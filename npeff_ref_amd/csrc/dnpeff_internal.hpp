@@ -169,6 +169,7 @@ struct tuning_t {
                                    // part, 2 = its far tail, -1 = the far tail where that pays (see use_nlists_tail)
   double t_lists = 0.0;            // A^T W in column blocks on component slices (1 = on)
   double nl_piece_cols = 32768.0;  // columns per piece of the slot lists
+  double nl_extra_mb = -1.0;       // MB the far tail's slot lists may take beyond their panel copy (-1: 1/128 of the device)
   double nl_lag = 0.0;             // pieces the workgroups of an XCD may be apart
   double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
   double gram_fold = 1.0;          // diagonal tiles of X^T X with the work their symmetry leaves (0 = all sixteen blocks)
@@ -285,6 +286,7 @@ struct dnpeff_csr {
   // prow[i] .. prow[i + 1] of pcol / pval), the others are in the slot lists nl
   int32_t tail_floor = 0;
   int64_t* prow = nullptr;
+  bool tail_declined = false;  // the far tail's slot lists did not fit the memory bound: it stays panels
   // after dnpeff_csr_split_dense_head: the dense block and the matrix of the remaining entries
   // (same shape, owned), which carries the derived structures the products use
   dn::slot_lists nl;

@@ -97,6 +97,7 @@ static const tuning_entry g_tuning_table[] = {
     {"topk_fast_cap", &tuning_t::topk_fast_cap}, {"verbose", &tuning_t::verbose},
     {"n_lists", &tuning_t::n_lists},             {"t_lists", &tuning_t::t_lists},
     {"nl_piece_cols", &tuning_t::nl_piece_cols}, {"nl_lag", &tuning_t::nl_lag},
+    {"nl_extra_mb", &tuning_t::nl_extra_mb},
     {"nl_spin", &tuning_t::nl_spin},             {"nl_wgs", &tuning_t::nl_wgs},
     {"gram_beside", &tuning_t::gram_beside},
     {"gram_fold", &tuning_t::gram_fold},
@@ -632,6 +633,7 @@ static void drop_panels(dnpeff_csr* A) {
 
 static void drop_derived(dnpeff_csr* A) {
   A->h_lists_valid = false;
+  A->tail_declined = false;
   drop_head(A);
   drop_panels(A);
   nlists_drop(A);
@@ -861,7 +863,7 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
     DN_TRY(nlists_build(S, r));
   } else {
     panel_plan plan = panel_policy(S, r);
-    plan.tail_lists = plan.coarse > 0 && plan.sweep_cols > 0 && use_nlists_tail(S, r);
+    plan.tail_lists = plan.coarse > 0 && plan.sweep_cols > 0 && use_nlists_tail(S, r) && !S->tail_declined;
     DN_TRY(csr_set_panels(S, plan));
     if (S->tail_floor > 0) {
       // Left to itself, the plan gives the lists what the panel copy of the same entries would
@@ -869,8 +871,11 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
       size_t free_b = 0, total_b = 0;
       DN_HIP(hipMemGetInfo(&free_b, &total_b));
       bool declined = false;
-      DN_TRY(nlists_build(S, r, S->tail_floor, tuning().n_lists < 0.0 ? (double)total_b / 128.0 : -1.0, &declined));
+      double bound = tuning().n_lists < 0.0 ? (double)total_b / 128.0 : -1.0;
+      if (tuning().nl_extra_mb >= 0.0) bound = tuning().nl_extra_mb * 1048576.0;
+      DN_TRY(nlists_build(S, r, S->tail_floor, bound, &declined));
       if (declined) {
+        S->tail_declined = true;  // (later calls must come to the same plan: the matrix may be consumed by then)
         plan.tail_lists = false;
         DN_TRY(csr_set_panels(S, plan));
       }

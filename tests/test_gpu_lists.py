@@ -207,3 +207,30 @@ def test_nmf_with_the_far_tail_on_slot_lists(tune):
     assert np.array_equal(nmf.loadWToHostSync(), W) and np.array_equal(nmf.loadHToHostSync(), H)
     nmf.close()
     A.close()
+
+
+def test_far_tail_stays_panels_when_its_lists_would_not_fit(tune):
+    """With no memory allowed beyond the panel copy the lists are declined, the tail stays plain
+    panels, and later plans of the same (by then consumed) matrix come to the same answer."""
+    r, n = 256, 2100
+    tune("n_lists", 2)
+    tune("nl_extra_mb", 0)
+    tune("panels", 8)
+    tune("sweep_bytes", 3000 * 4 * r)
+    tune("sweep_min", 40)
+    m_full, k, iters, eps, seed = 100000, 2000, 5, 1e-12, 79
+    A, norms = d.Csr.synth(n, m_full, k_fixed=k, zipf_s=1.3, seed=seed)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    rp, ci, va = A.download()
+    nmf = d.MuNmf(A, d.MuNmfParams(rank=r, max_iters=iters, eps=eps, seed=seed, log_every=5), consume_matrix=True)
+    info = A.products_info()
+    assert info["tail_floor"] == 0 and info["list_entries"] == 0 and info["swept_pieces"] > 0 and info["plain"] > 1, info
+    nmf.initialize()
+    W0, H0 = nmf.loadWToHostSync(), nmf.loadHToHostSync()
+    nmf.run(log=lambda s: None)
+    W64, H64, _ = orc.nmf_f64(rp, ci, va, A.n_cols, W0, H0, np.float32(eps), iters, 5)
+    assert np.linalg.norm(nmf.loadWToHostSync() - W64) / np.linalg.norm(W64) < 1e-4
+    assert A.products_info() == info
+    nmf.close()
+    A.close()
