@@ -234,3 +234,40 @@ def test_far_tail_stays_panels_when_its_lists_would_not_fit(tune):
     assert A.products_info() == info
     nmf.close()
     A.close()
+
+
+def test_far_tail_lists_with_ragged_empty_and_tail_only_rows(tune):
+    """Rows of 16 ... 4,096 entries, two empty rows, one row with entries in the far tail only and
+    one with none there: the panel copy without the tail and the lists must split every row where
+    its entries say, wherever they stand in the row."""
+    r = 256
+    _tail_plan(tune, r, piece_cols=1500, sweep_min=12)
+    rng = np.random.default_rng(11)
+    n, m_full = 420, 60000
+    rowptr, colind, vals, _ = d.synth_pef_host(n, m_full, k_fixed=0, k_min=16, k_max=4096, zipf_s=1.1, seed=21)
+    keep = np.ones(len(colind), dtype=bool)
+    row_of = np.repeat(np.arange(n), np.diff(rowptr))
+    keep[(row_of == 1) | (row_of == n - 1)] = False                 # empty rows
+    keep[(row_of == 5) & (colind < 30000)] = False                  # far columns only
+    keep[(row_of == 6) & (colind >= 2000)] = False                  # near columns only
+    colind, vals = colind[keep], vals[keep]
+    rowptr = np.concatenate([[0], np.cumsum(np.bincount(row_of[keep], minlength=n))]).astype(np.int64)
+    A = d.Csr.from_host(rowptr, colind, vals, m_full)
+    H = rng.random((m_full, r)).astype(np.float32)
+    dH, dN = d.DeviceArray.from_numpy(H), d.DeviceArray((n, r))
+    d.op_spmm_n(A, r, dH, dN)
+    info = A.products_info()
+    assert info["tail_floor"] > 0 and info["swept_pieces"] > 0, info
+    assert info["list_entries"] == int((colind >= info["tail_floor"]).sum())
+    assert 2000 < info["tail_floor"] <= 30000  # rows 5 and 6 lie on one side each
+    N = dN.numpy()
+    want = orc.spmm_n_f64(rowptr, colind, vals, H)
+    assert _row_rel(N[[i for i in range(n) if i not in (1, n - 1)]].astype(np.float64),
+                    want[[i for i in range(n) if i not in (1, n - 1)]]) < TOL
+    assert np.all(N[1] == 0) and np.all(N[n - 1] == 0)
+    for i in (0, 1, 5, 6, n - 1):
+        cols, got = A.get_row(i)
+        o, ow = np.argsort(cols, kind="stable"), np.argsort(colind[rowptr[i]:rowptr[i + 1]], kind="stable")
+        assert np.array_equal(cols[o], colind[rowptr[i]:rowptr[i + 1]][ow])
+        assert np.array_equal(got[o], vals[rowptr[i]:rowptr[i + 1]][ow])
+    A.close()
