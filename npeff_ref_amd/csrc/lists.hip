@@ -7,7 +7,7 @@
 // is eight times smaller and stays in its own L2:
 //
 //   A H^T  (k_spmm_n_lists): XCD x sums components [32 x, 32 x + 32) of every row of the result.
-//     The running sums of all rows live in the LDS of the XCD's CUs (a wave slot owns up to 72
+//     The running sums of all rows live in the LDS of the XCD's CUs (a wave slot owns up to 80
 //     rows, 512 slots per XCD), and all slots walk the columns in the same order, piece by piece
 //     (a piece: 32,768 columns, 4 MB of 128-byte row slices of H), so that a row slice of H is
 //     fetched from HBM once and found in the L2 by the other rows that use it.  This is how the
@@ -41,7 +41,7 @@ namespace dn {
 constexpr int NL_WAVES = 8;                      // waves per workgroup of the A H^T kernel
 constexpr int NL_WGS_MAX = 96;                   // its workgroups per XCD: two (or three) per CU
 constexpr int NL_ROW_BYTES = 128;                // one row of running sums in LDS: 32 floats
-constexpr int NL_RPW_MAX = 72;                   // rows per wave slot (8 x 72 x 128 bytes <= half the LDS)
+constexpr int NL_RPW_MAX = 80;                   // rows per wave slot (8 x 80 x 128 bytes = half the LDS)
 constexpr int NL_SLICE = 32;                     // components per slice
 constexpr int NL_MAX_SLOTS = 4096;
 constexpr int NL_MAX_PIECES = 16000;             // (the builder keeps one counter per piece in LDS)
