@@ -422,6 +422,7 @@ def run_nmf(d, args, cfg):
         except d.DnpeffError as e:
             log(f"products on the fp32 matrix cores: not measured ({e})")
         d.tuning_set("split_bf16", 1)
+    sparse_plan = A.products_info()
     nmf.close()
     A.close()
 
@@ -467,7 +468,8 @@ def run_nmf(d, args, cfg):
                    "n_features_kept": m, "nnz": z, "nnz_per_row": cfg["k"] or [cfg["kmin"], cfg["kmax"]],
                    "zipf_s": cfg["s"], "rank": r, "eps": args.eps, "seed": args.seed,
                    "dense_head_columns": n_dense, "nnz_sparse_part": z_sparse, "tiled_H_update": tiled,
-                   "H_tile_columns": tile_cols, "device_memory_used_gb": (total - free1) / 1e9,
+                   "H_tile_columns": tile_cols, "sparse_part_of_A_Ht": sparse_plan,
+                   "device_memory_used_gb": (total - free1) / 1e9,
                    "device_memory_total_gb": total / 1e9},
         "roofline": roofline,
         "roofline_gather_model": gather_model,
