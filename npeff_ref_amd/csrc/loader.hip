@@ -868,11 +868,14 @@ int csr_ensure_products(dnpeff_csr* A, int r) {
     if (S->tail_floor > 0) {
       // Left to itself, the plan gives the lists what the panel copy of the same entries would
       // take plus half of the memory that the plan keeps free; beyond that the tail stays panels.
-      size_t free_b = 0, total_b = 0;
-      DN_HIP(hipMemGetInfo(&free_b, &total_b));
       bool declined = false;
-      double bound = tuning().n_lists < 0.0 ? (double)total_b / 128.0 : -1.0;
-      if (tuning().nl_extra_mb >= 0.0) bound = tuning().nl_extra_mb * 1048576.0;
+      double bound = -1.0;
+      if (!(S->nl.pairs && S->nl.floor_col == S->tail_floor)) {  // (lists that exist are not judged again)
+        size_t free_b = 0, total_b = 0;
+        DN_HIP(hipMemGetInfo(&free_b, &total_b));
+        if (tuning().n_lists < 0.0) bound = (double)total_b / 128.0;
+        if (tuning().nl_extra_mb >= 0.0) bound = tuning().nl_extra_mb * 1048576.0;
+      }
       DN_TRY(nlists_build(S, r, S->tail_floor, bound, &declined));
       if (declined) {
         S->tail_declined = true;  // (later calls must come to the same plan: the matrix may be consumed by then)
