@@ -46,6 +46,9 @@ struct AbtOperand {
       for (int q = 0; q < 4; q++) r[q] = *reinterpret_cast<const f32x4*>(p + q * ld);
     }
   }
+  // PLANE: bytes between the parts of the tile (a tile of 256 rows from a workgroup of 512 has
+  // planes of twice the size)
+  template <int PLANE = ABT_PLANE>
   __device__ __forceinline__ void commit(unsigned char* planes) const {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
@@ -61,8 +64,8 @@ struct AbtOperand {
         dst = planes + (row4 + q) * ABT_LD + 2 * kb;
       }
       *reinterpret_cast<bf16x4*>(dst) = h;
-      *reinterpret_cast<bf16x4*>(dst + ABT_PLANE) = m;
-      *reinterpret_cast<bf16x4*>(dst + 2 * ABT_PLANE) = l;
+      *reinterpret_cast<bf16x4*>(dst + PLANE) = m;
+      *reinterpret_cast<bf16x4*>(dst + 2 * PLANE) = l;
     }
   }
 };
@@ -251,6 +254,102 @@ __device__ __forceinline__ void gram_diag_mainloop(const float* __restrict__ src
         mfma_tile();
         __syncthreads();  // every wave is done with the planes
         oa[(u + 1) % STAGES].commit(ab);
+        fetch((u + 1) % STAGES, t + u + 1 + STAGES);
+        __syncthreads();
+      }
+    }
+  }
+}
+
+// A diagonal square of 256 columns of X^T X in one workgroup of eight waves: the 8 x 8 blocks of
+// 32 x 32 with the work the symmetry leaves, and every element of X fetched, split and stored
+// once for all of them.  Wave w owns block row w of the operand tile as first operand and forms
+//   the blocks (w, w + 1), (w, w + 2), (w, w + 3) (indices modulo 8; six products each),
+//   the diagonal block (w, w) as Q and P apart (four products, see gram_diag_mainloop),
+//   half of the block (w, w + 4): waves 0-3 the products h h, h m, m h, waves 4-7 (which hold the
+//   block as (w, w - 4), the transpose) h l, l h, m m;
+// 25 matrix instructions per 16 contraction elements and wave, where all 64 blocks with six
+// products take 48.  The planes are kept twice: the next tile is stored while slower waves still
+// read the current one, and one barrier per tile is enough.
+// acc: [0..2] = blocks (w, w + 1 .. w + 3), [3] = Q, [4] = P, [5] = the half block.
+constexpr int ABT_PLANE2 = 256 * ABT_LD;
+constexpr int ABT_LDS_PAIR = 2 * 3 * ABT_PLANE2;
+
+template <int STAGES>
+__device__ __forceinline__ void gram_pair_mainloop(const float* __restrict__ src, int64_t ld,
+                                                   int64_t first, int64_t stride, int64_t n_tiles,
+                                                   unsigned char* ab, abt_acc16 (&acc)[6]) {
+  static_assert(STAGES == 1 || STAGES == 2, "one or two tiles in registers");
+  if (n_tiles <= 0) return;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l32 = lane & 31, half = lane >> 5;
+  const bool low = wave < 4;
+  AbtOperand<true> oa[STAGES];
+  auto fetch = [&](int s, int64_t t) {
+    const int64_t k0 = (first + (t < n_tiles ? t : n_tiles - 1) * stride) * ABT_KB;
+    oa[s].fetch(src, ld, k0);
+  };
+  const int lane_at = l32 * ABT_LD + 16 * half;
+  int row_at[5];
+#pragma unroll
+  for (int k = 0; k < 5; k++) row_at[k] = lane_at + 32 * ((wave + k) & 7) * ABT_LD;
+  auto planes = [&](const unsigned char* p, bf16x8& h, bf16x8& m, bf16x8& l) {
+    h = *reinterpret_cast<const bf16x8*>(p);
+    m = *reinterpret_cast<const bf16x8*>(p + ABT_PLANE2);
+    l = *reinterpret_cast<const bf16x8*>(p + 2 * ABT_PLANE2);
+  };
+  auto mfma_tile = [&](const unsigned char* buf) {
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+      bf16x8 xh, xm, xl, yh, ym, yl;
+      planes(buf + row_at[0] + 32 * st, xh, xm, xl);
+      planes(buf + row_at[1] + 32 * st, yh, ym, yl);
+      acc[0] = DN_MFMA_B16(xh, yh, acc[0]);
+      acc[3] = DN_MFMA_B16(xh, xh, acc[3]);
+      acc[0] = DN_MFMA_B16(xh, ym, acc[0]);
+      acc[4] = DN_MFMA_B16(xh, xm, acc[4]);
+      acc[0] = DN_MFMA_B16(xm, yh, acc[0]);
+      acc[3] = DN_MFMA_B16(xm, xm, acc[3]);
+      acc[0] = DN_MFMA_B16(xh, yl, acc[0]);
+      acc[4] = DN_MFMA_B16(xh, xl, acc[4]);
+      acc[0] = DN_MFMA_B16(xl, yh, acc[0]);
+      acc[0] = DN_MFMA_B16(xm, ym, acc[0]);
+#pragma unroll
+      for (int k = 2; k < 4; k++) {
+        planes(buf + row_at[k] + 32 * st, yh, ym, yl);
+        acc[k - 1] = DN_MFMA_B16(xh, yh, acc[k - 1]);
+        acc[k - 1] = DN_MFMA_B16(xh, ym, acc[k - 1]);
+        acc[k - 1] = DN_MFMA_B16(xm, yh, acc[k - 1]);
+        acc[k - 1] = DN_MFMA_B16(xh, yl, acc[k - 1]);
+        acc[k - 1] = DN_MFMA_B16(xl, yh, acc[k - 1]);
+        acc[k - 1] = DN_MFMA_B16(xm, ym, acc[k - 1]);
+      }
+      planes(buf + row_at[4] + 32 * st, yh, ym, yl);
+      if (low) {
+        acc[5] = DN_MFMA_B16(xh, yh, acc[5]);
+        acc[5] = DN_MFMA_B16(xh, ym, acc[5]);
+        acc[5] = DN_MFMA_B16(xm, yh, acc[5]);
+      } else {
+        acc[5] = DN_MFMA_B16(xh, yl, acc[5]);
+        acc[5] = DN_MFMA_B16(xl, yh, acc[5]);
+        acc[5] = DN_MFMA_B16(xm, ym, acc[5]);
+      }
+    }
+  };
+  // At the top of tile t: buffer t % 2 holds tile t, and register stage (t + 1 + s) % STAGES holds
+  // tile t + 1 + s.  Buffer (t + 1) % 2 was last read for tile t - 1, before that tile's barrier.
+  fetch(0, 0);
+  oa[0].template commit<ABT_PLANE2>(ab);
+#pragma unroll
+  for (int s = 0; s < STAGES; s++) fetch((1 + s) % STAGES, 1 + s);
+  __syncthreads();
+  for (int64_t t = 0; t < n_tiles; t += STAGES) {
+#pragma unroll
+    for (int u = 0; u < STAGES; u++) {
+      if (t + u < n_tiles) {
+        const int cur = (int)((t + u) & 1);
+        mfma_tile(ab + cur * (3 * ABT_PLANE2));
+        oa[(u + 1) % STAGES].template commit<ABT_PLANE2>(ab + (cur ^ 1) * (3 * ABT_PLANE2));
         fetch((u + 1) % STAGES, t + u + 1 + STAGES);
         __syncthreads();
       }

@@ -340,21 +340,26 @@ static int64_t gram_tiles_slices(int64_t rows, int r) {
 // The split-operand kernel runs the diagonal tile pairs and the others as two launches (a
 // diagonal pair fetches and splits one tile, not two), each with the slices that fill the 2
 // workgroup slots per CU once.
-static void gram_b16_slices(int64_t rows, int r, int64_t* s_diag, int64_t* s_off) {
+// paired: the diagonal tiles go two and two as squares of 256 columns (one workgroup of eight
+// waves per CU), and the other launch takes the tile pairs that lie outside those squares.
+static bool gram_paired(int r) { return tuning().gram_fold >= 2 && r % 256 == 0; }
+static void gram_b16_slices(int64_t rows, int r, int64_t* s_diag, int64_t* s_off, bool paired = false) {
   const int64_t t = r / 128, slots = 2 * (int64_t)n_cus(), k_tiles = rows / 32;
-  int64_t d = slots / t, o = t > 1 ? slots / (t * (t - 1) / 2) : 0;
+  const int64_t n_off = t * (t - 1) / 2 - (paired ? t / 2 : 0);
+  int64_t d = slots / t, o = n_off > 0 ? slots / n_off : 0;  // (paired: t / 2 squares, one slot per CU)
   if (d < 1) d = 1;
-  if (t > 1 && o < 1) o = 1;
+  if (n_off > 0 && o < 1) o = 1;
   if (d > k_tiles) d = k_tiles;
   if (o > k_tiles) o = k_tiles;
   *s_diag = d < 1 ? 1 : d;
-  *s_off = t > 1 ? (o < 1 ? 1 : o) : 0;
+  *s_off = n_off > 0 ? (o < 1 ? 1 : o) : 0;
 }
 
 int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
-  int64_t d, o;
+  int64_t d, o, dp, op;
   gram_b16_slices(rows, r, &d, &o);
-  const int64_t s = std::max(gram_tiles_slices(rows, r), std::max(d, o));
+  gram_b16_slices(rows, r, &dp, &op, true);
+  const int64_t s = std::max(std::max(gram_tiles_slices(rows, r), std::max(d, o)), std::max(dp, op));
   return (s + 1) * (int64_t)r * r;
 }
 
@@ -362,16 +367,20 @@ int64_t gram_tiles_workspace_floats(int64_t rows, int r) {
 // one more term of every tile (the last rows, from the fp32 kernel).
 __global__ void __launch_bounds__(256)
     k_gram_tiles_reduce(const float* __restrict__ ws, int64_t s_diag, int64_t s_off, int64_t extra, int r,
-                        bool folded, float* __restrict__ G) {
+                        int folded, float* __restrict__ G) {
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= r * r) return;
   const int a = e / r, b = e % r;
-  if ((a >> 7) > (b >> 7) || ((a >> 7) == (b >> 7) && a > b)) return;  // upper triangle only
+  if (a > b) return;  // upper triangle only
   double s = 0.0;
   const int64_t stride = (int64_t)r * r;
-  const int64_t slices = (a >> 7) == (b >> 7) ? s_diag : s_off;
-  if (folded && (a >> 5) == (b >> 5)) {
-    // a diagonal block of 32 x 32 from k_gram_diag_b16: the stored block plus its transpose
+  // folded = 1: diagonal tiles of 128 from k_gram_diag_b16; 2: diagonal squares of 256 from
+  // k_gram_pair_b16, where the block four block columns to the right of the diagonal comes in
+  // two halves, one of them stored transposed below the diagonal
+  const bool own = folded == 2 ? (a >> 8) == (b >> 8) : (a >> 7) == (b >> 7);
+  const int64_t slices = own ? s_diag : s_off;
+  if (folded && ((a >> 5) == (b >> 5) || (folded == 2 && own && (b >> 5) - (a >> 5) == 4))) {
+    // the stored block plus (the stored block at the mirrored place) transposed
     const int et = b * r + a;
     for (int64_t sl = 0; sl < slices; sl++)
       s += (double)ws[sl * stride + e] + (double)ws[sl * stride + et];
@@ -387,24 +396,29 @@ __global__ void __launch_bounds__(256)
 // tiles of 32 rows only; the caller adds the last rows.
 // DIAG: grid.x numbers the diagonal tiles; otherwise the tile pairs (ti < tj) row by row: every
 // workgroup of the grid works.
+// paired (not DIAG): without the pairs (2 g, 2 g + 1), which k_gram_pair_b16 covers.
 template <bool DIAG>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     k_gram_tiles_b16(const float* __restrict__ X, int64_t k_tiles, int r, int n_tiles_side,
-                     float* __restrict__ out) {
+                     float* __restrict__ out, bool paired) {
   extern __shared__ __align__(16) unsigned char ab[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
   int ti = blockIdx.x, tj = blockIdx.x;
   if (!DIAG) {
-    int p = blockIdx.x, row_len = n_tiles_side - 1;
+    int p = blockIdx.x;
     ti = 0;
-    while (p >= row_len) {
+    for (;;) {
+      const int first = ti + 1 + ((paired && !(ti & 1)) ? 1 : 0), row_len = n_tiles_side - first;
+      if (p < row_len || ti >= n_tiles_side - 1) {
+        tj = first + p;
+        break;
+      }
       p -= row_len;
       ti++;
-      row_len--;
     }
-    tj = ti + 1 + p;
+    if (tj >= n_tiles_side) return;  // (a grid larger than the pairs: not launched)
   }
   const int64_t S = gridDim.z, z = blockIdx.z;
   const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
@@ -466,10 +480,55 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
+// A diagonal square of 256 columns (gram_pair_mainloop): its 36 upper blocks of 32 x 32 are
+// stored, those on the diagonal as Q / 2 + P; blocks that a wave holds as (w, j) with j < w are
+// stored transposed at (j, w); the half block that waves 4-7 hold of (w - 4, w) stays as it is,
+// below the diagonal at (w, w - 4), and the reduction adds its transpose to the other half.
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    k_gram_pair_b16(const float* __restrict__ X, int64_t k_tiles, int r, float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char ab[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int g = blockIdx.x;
+  const int64_t S = gridDim.z, z = blockIdx.z;
+  const int64_t n_my = z < k_tiles ? (k_tiles - z + S - 1) / S : 0;
+  acc16 acc[6];
+#pragma unroll
+  for (int b = 0; b < 6; b++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[b][v] = 0.0f;
+  gram_pair_mainloop<ABT_STAGES_GRAM>(X + 256 * g, r, z, S, n_my, ab, acc);
+  float* square = out + ((int64_t)z * r + 256 * g) * r + 256 * g;
+  // element (8 (v / 4) + v % 4 + 4 half, l32) of block (bi, bj)
+  auto store = [&](int bi, int bj, const acc16& c) {
+    float* base = square + (int64_t)(32 * bi + 4 * half) * r + 32 * bj + l32;
+#pragma unroll
+    for (int v = 0; v < 16; v++) base[(int64_t)(8 * (v >> 2) + (v & 3)) * r] = c[v];
+  };
+  auto store_transposed = [&](int bi, int bj, const acc16& c) {  // the block (bi, bj) to the place (bj, bi)
+    float* base = square + (int64_t)(32 * bj + l32) * r + 32 * bi + 4 * half;
+#pragma unroll
+    for (int v = 0; v < 16; v++) base[8 * (v >> 2) + (v & 3)] = c[v];
+  };
+#pragma unroll
+  for (int k = 1; k < 4; k++) {
+    const int bj = (wave + k) & 7;
+    if (bj > wave)
+      store(wave, bj, acc[k - 1]);
+    else
+      store_transposed(wave, bj, acc[k - 1]);
+  }
+  acc16 d;
+#pragma unroll
+  for (int v = 0; v < 16; v++) d[v] = 0.5f * acc[3][v] + acc[4][v];
+  store(wave, wave, d);
+  store(wave, (wave + 4) & 7, acc[5]);
+}
+
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace) {
   const int t = r / 128;
   int64_t s_diag, s_off, extra = -1;
-  bool folded = false;
+  int folded = 0;
   if (use_split_bf16() && rows >= ABT_KB) {
     static bool attr_set = false;
     if (!attr_set) {
@@ -479,22 +538,29 @@ int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* work
                                  hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
       DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_diag_b16),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
+      DN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gram_pair_b16),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS_PAIR));
       attr_set = true;
     }
     // whole contraction tiles on the bf16 matrix cores, the last rows (fewer than 32) as one
     // more slice through the fp32 kernel
     const int64_t k_tiles = rows / ABT_KB, whole = k_tiles * ABT_KB;
-    gram_b16_slices(rows, r, &s_diag, &s_off);
-    folded = tuning().gram_fold != 0;
-    if (folded)
+    const bool paired = gram_paired(r);
+    gram_b16_slices(rows, r, &s_diag, &s_off, paired);
+    folded = paired ? 2 : tuning().gram_fold != 0 ? 1 : 0;
+    const int n_off = t * (t - 1) / 2 - (paired ? t / 2 : 0);
+    if (paired)
+      hipLaunchKernelGGL(k_gram_pair_b16, dim3((unsigned)(t / 2), 1, (unsigned)s_diag), dim3(512), ABT_LDS_PAIR,
+                         stream(), X, k_tiles, r, workspace);
+    else if (folded)
       hipLaunchKernelGGL(k_gram_diag_b16, dim3((unsigned)t, 1, (unsigned)s_diag), dim3(256), ABT_LDS, stream(),
                          X, k_tiles, r, workspace);
     else
       hipLaunchKernelGGL(k_gram_tiles_b16<true>, dim3((unsigned)t, 1, (unsigned)s_diag), dim3(256), ABT_LDS,
-                         stream(), X, k_tiles, r, t, workspace);
-    if (t > 1)
-      hipLaunchKernelGGL(k_gram_tiles_b16<false>, dim3((unsigned)(t * (t - 1) / 2), 1, (unsigned)s_off),
-                         dim3(256), ABT_LDS, stream(), X, k_tiles, r, t, workspace);
+                         stream(), X, k_tiles, r, t, workspace, false);
+    if (n_off > 0)
+      hipLaunchKernelGGL(k_gram_tiles_b16<false>, dim3((unsigned)n_off, 1, (unsigned)s_off),
+                         dim3(256), ABT_LDS, stream(), X, k_tiles, r, t, workspace, paired);
     DN_LAUNCH_CHECK();
     if (whole < rows) {
       extra = std::max(s_diag, s_off);

@@ -84,12 +84,15 @@ def test_gram(rows, r):
     assert np.array_equal(G, G.T) or _rel(G, G.T.astype(np.float64)) < 1e-6
 
 
-@pytest.mark.parametrize("fold", [1, 0])
-@pytest.mark.parametrize("rows,r", [(4096, 256), (20011, 256), (3000, 384), (2500, 1024)])
+@pytest.mark.parametrize("fold", [2, 1, 0])
+@pytest.mark.parametrize("rows,r", [(4096, 256), (20011, 256), (3000, 384), (2500, 1024), (9000, 512), (31, 256),
+                                    (64, 512)])
 def test_gram_diagonal_tiles_with_and_without_their_symmetry(rows, r, fold, tune):
     """X^T X at the ranks that run on tiles, with signed entries over eight decades (a partial
     product taken from the wrong side of the diagonal, or left out, shows at 2^-8 or 2^-16 of the
-    element), the diagonal tiles folded (ten blocks, four products on the diagonal ones) and not."""
+    element): the diagonal tiles two and two as squares of 256 columns in one workgroup (36 of 64
+    blocks, a block in two halves; at ranks that are multiples of 256), each by itself with its
+    symmetry used (ten blocks, four products on the diagonal ones), and plain."""
     tune("gram_fold", fold)
     rng = np.random.default_rng(rows + r + fold)
     X = (rng.standard_normal((rows, r)) * 10.0 ** rng.uniform(-4, 4, size=(1, r))).astype(np.float32)
