@@ -77,8 +77,9 @@ int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int
 /* Switches for experiments and for tests that must reach a particular code path; no counterpart
  * in the reference.  Names: dense_fill, panels, sweep_bytes, sweep_min, sweep_waves, sweep_lag,
  * sweep_spin, spmm_t_slices, split_bf16, fused_gram, h_tile_mb, tiled_h, topk_fast_cap, verbose,
- * gram_beside (H^T H of the W update on a second stream beside A H^T), gram_fold (0: diagonal
- * tiles of X^T X without the use of their symmetry), n_lists (A H^T from slot lists on component slices of 32: -1 =
+ * gram_beside (H^T H of the W update on a second stream beside A H^T), gram_fold (2: X^T X with
+ * its diagonal squares of 256 columns each in one workgroup where the rank is a multiple of 256;
+ * 1: diagonal tiles of 128 columns with their symmetry used; 0: without), n_lists (A H^T from slot lists on component slices of 32: -1 =
  * the far tail of the sparse part where that was measured to pay, 2 = wherever possible, 1 = the
  * whole sparse part, 0 = never), t_lists (1: A^T W in column blocks on such slices), nl_piece_cols,
  * nl_lag, nl_spin, nl_wgs (their piece size, lock step and launch shape), nl_extra_mb (memory the
