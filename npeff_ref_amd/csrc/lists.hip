@@ -35,6 +35,7 @@
 #include <cstring>
 #include <type_traits>
 #include <utility>
+#include <vector>
 
 namespace dn {
 
@@ -647,6 +648,29 @@ int nlists_build(dnpeff_csr* S, int r, int32_t floor_col, double max_extra_bytes
   hipLaunchKernelGGL(k_nl_slot_scan, dim3((unsigned)n_slots), dim3(256), 0, st, nbat.p, n_pieces, L.off);
   DN_LAUNCH_CHECK();
   DN_HIP(hipStreamSynchronize(st));
+  if (tuning().verbose >= 2.0) {  // how far the lock step of an XCD's waves is from the mean work
+    std::vector<uint32_t> hb((size_t)n_slots * n_pieces);
+    DN_HIP(hipMemcpy(hb.data(), nbat.p, hb.size() * 4, hipMemcpyDeviceToHost));
+    double sum = 0, sum_max = 0, sum_wgmax = 0;
+    for (int p = 0; p < n_pieces; p++) {
+      uint32_t mx = 0;
+      double wg = 0;
+      for (int s0 = 0; s0 < n_slots; s0 += NL_WAVES) {
+        uint32_t m8 = 0;
+        for (int w = 0; w < NL_WAVES; w++) {
+          const uint32_t v = hb[(size_t)(s0 + w) * n_pieces + p];
+          sum += v;
+          m8 = v > m8 ? v : m8;
+        }
+        wg += m8;
+        mx = m8 > mx ? m8 : mx;
+      }
+      sum_max += mx;
+      sum_wgmax += wg / (n_slots / NL_WAVES);
+    }
+    std::fprintf(stderr, "dnpeff: slot lists: batches per slot %.0f, sum over pieces of the longest slot %.0f, of the mean over workgroups of their longest wave %.0f\n",
+                 sum / n_slots, sum_max, sum_wgmax);
+  }
   nbat.reset();
   // batches of the slots -> first batch of each slot
   std::vector<uint32_t> tot((size_t)n_slots);
