@@ -85,7 +85,7 @@ def test_gram(rows, r):
 
 
 @pytest.mark.parametrize("fold", [2, 1, 0])
-@pytest.mark.parametrize("rows,r", [(4096, 256), (20011, 256), (3000, 384), (2500, 1024), (9000, 512), (31, 256),
+@pytest.mark.parametrize("rows,r", [(4096, 256), (20011, 256), (3000, 384), (2500, 1024), (9000, 512), (1500, 768), (31, 256),
                                     (64, 512)])
 def test_gram_diagonal_tiles_with_and_without_their_symmetry(rows, r, fold, tune):
     """X^T X at the ranks that run on tiles, with signed entries over eight decades (a partial
