@@ -166,6 +166,106 @@ __device__ __forceinline__ void abt_mainloop(const float* __restrict__ a_src, in
   }
 }
 
+// The product of abt_mainloop for operands with the contraction index fast, on planes without
+// padding (64 bytes per row: 48 KB for the six planes, so that three workgroups fit a CU): the
+// four 16-byte pieces of a row are stored at piece ^ (row / 4 % 4), which spreads the sixteen rows
+// that a 16-byte LDS read instruction takes at a time over all banks.  One tile travels in
+// registers (a third workgroup per CU hides what a second stage would).
+constexpr int ABT_LD64 = 64;
+constexpr int ABT_PLANE64 = 128 * ABT_LD64;
+constexpr int ABT_LDS64 = 6 * ABT_PLANE64;
+
+__device__ __forceinline__ void abt_fetch_kfast(f32x4 (&r)[4], const float* __restrict__ src, int64_t ld, int64_t k0) {
+  const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
+#pragma unroll
+  for (int q = 0; q < 4; q++) r[q] = *reinterpret_cast<const f32x4*>(src + (int64_t)(fr + 32 * q) * ld + k0 + fk);
+}
+__device__ __forceinline__ void abt_commit64(const f32x4 (&r)[4], unsigned char* planes) {
+  const int fr = threadIdx.x >> 3, fk = 4 * (threadIdx.x & 7);
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    bf16x4 h, m, l;
+    split3(r[q], h, m, l);
+    const int row = fr + 32 * q;
+    unsigned char* dst = planes + row * ABT_LD64 + (((fk >> 3) ^ ((row >> 2) & 3)) << 4) + 2 * (fk & 7);
+    *reinterpret_cast<bf16x4*>(dst) = h;
+    *reinterpret_cast<bf16x4*>(dst + ABT_PLANE64) = m;
+    *reinterpret_cast<bf16x4*>(dst + 2 * ABT_PLANE64) = l;
+  }
+}
+
+__device__ __forceinline__ void abt_mainloop64(const float* __restrict__ a_src, int64_t lda,
+                                               const float* __restrict__ b_src, int64_t ldb, int n_tiles,
+                                               unsigned char* ab, abt_acc16 (&acc)[2][2]) {
+  if (n_tiles <= 0) return;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l32 = lane & 31, half = lane >> 5, wm = wave >> 1, wn = wave & 1;
+  f32x4 oa[4], ob[4];
+  auto fetch = [&](int t) {
+    const int64_t k0 = (int64_t)(t < n_tiles ? t : n_tiles - 1) * ABT_KB;
+    abt_fetch_kfast(oa, a_src, lda, k0);
+    abt_fetch_kfast(ob, b_src, ldb, k0);
+  };
+  const int swz = (l32 >> 2) & 3;
+  const unsigned char* a_row = ab + (64 * wm + l32) * ABT_LD64;
+  const unsigned char* b_row = ab + 3 * ABT_PLANE64 + (64 * wn + l32) * ABT_LD64;
+  auto mfma_tile = [&]() {
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+      const int at = ((2 * st + half) ^ swz) << 4;
+      bf16x8 ah[2], am[2], al[2], bh[2], bm[2], bl[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const unsigned char* pa = a_row + 32 * i * ABT_LD64 + at;
+        ah[i] = *reinterpret_cast<const bf16x8*>(pa);
+        am[i] = *reinterpret_cast<const bf16x8*>(pa + ABT_PLANE64);
+        al[i] = *reinterpret_cast<const bf16x8*>(pa + 2 * ABT_PLANE64);
+        const unsigned char* pb = b_row + 32 * i * ABT_LD64 + at;
+        bh[i] = *reinterpret_cast<const bf16x8*>(pb);
+        bm[i] = *reinterpret_cast<const bf16x8*>(pb + ABT_PLANE64);
+        bl[i] = *reinterpret_cast<const bf16x8*>(pb + 2 * ABT_PLANE64);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bm[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(ah[i], bl[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(al[i], bh[j], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = DN_MFMA_B16(am[i], bm[j], acc[i][j]);
+    }
+  };
+  fetch(0);
+  abt_commit64(oa, ab);
+  abt_commit64(ob, ab + 3 * ABT_PLANE64);
+  fetch(1);
+  __syncthreads();
+  for (int t = 0; t < n_tiles; t++) {
+    mfma_tile();
+    __syncthreads();
+    abt_commit64(oa, ab);
+    abt_commit64(ob, ab + 3 * ABT_PLANE64);
+    fetch(t + 2);
+    __syncthreads();
+  }
+}
+
 // A diagonal tile of X^T X (128 columns of X against themselves) with the work that its symmetry
 // leaves: of the 4 x 4 blocks of 32 x 32 only the ten with block row <= block column are formed,
 // and a block on the diagonal needs four of the six partial products, because h^T m and m^T h

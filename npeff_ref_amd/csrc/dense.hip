@@ -1056,6 +1056,71 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   finish(3, pn[1], px[1]);
 }
 
+// The same with three workgroups per CU (abt_mainloop64).
+template <bool WITH_D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
+    k_xg_mu_tile_b16_w3(const float* __restrict__ X, const float* __restrict__ Gt, const float* num,
+                     float eps, int64_t n_row_tiles, int r, int n_chunks, float* out,
+                     float* __restrict__ D_out) {
+  extern __shared__ __align__(16) unsigned char ab[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  // Workgroups are dealt to the 8 XCDs round-robin by their number; the column chunks of one row
+  // tile are numbered 8 apart so that they share an XCD, i.e. an L2, and X comes in once.
+  const int64_t grp = blockIdx.x / (8 * n_chunks);
+  const int rem = (int)(blockIdx.x % (8 * n_chunks));
+  const int64_t tile = grp * 8 + rem % 8;
+  if (tile >= n_row_tiles) return;
+  const int n0 = (rem / 8) * 128;
+  const int64_t row0 = tile * 128;
+
+  // element (i, j, v): row 64 wm + 32 i + 8 (v / 4) + 4 half + v % 4, column n0 + 64 wn + 32 j + l32
+  const int64_t t0 = (row0 + 64 * wm + 4 * half) * (int64_t)r + n0 + 64 * wn;
+  const float* tnum = num + t0;
+  const float* tx = X + t0;
+  float* tout = out + t0;
+  float* tD = WITH_D ? D_out + t0 : nullptr;
+  float pn[2][16], px[2][16];
+  auto request = [&](int blk, float (&n_)[16], float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int64_t off = (32 * i + 8 * (v >> 2) + (v & 3)) * (int64_t)r + 32 * j + l32;
+      n_[v] = tnum[off];
+      x_[v] = tx[off];
+    }
+  };
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+  abt_mainloop64(X + row0 * r, r, Gt + (int64_t)n0 * r, r, r / ABT_KB, ab, acc);
+
+  auto finish = [&](int blk, const float (&n_)[16], const float (&x_)[16]) {
+    const int i = blk >> 1, j = blk & 1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int64_t off = (32 * i + 8 * (v >> 2) + (v & 3)) * (int64_t)r + 32 * j + l32;
+      const float d = acc[i][j][v];
+      const float q = mu_quotient(n_[v], d + eps);
+      tout[off] = x_[v] * q;
+      if (WITH_D) tD[off] = d;
+    }
+  };
+  request(0, pn[0], px[0]);
+  request(1, pn[1], px[1]);
+  finish(0, pn[0], px[0]);
+  request(2, pn[0], px[0]);
+  finish(1, pn[1], px[1]);
+  request(3, pn[1], px[1]);
+  finish(2, pn[0], px[0]);
+  finish(3, pn[1], px[1]);
+}
+
 // G transposed for the split-operand update: a buffer that grows to the largest rank seen and
 // lives until the process ends (one host thread drives the library).
 static float* g_gt = nullptr;
@@ -1086,7 +1151,14 @@ static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const floa
     const int64_t wgs = ceil_div(tiles, 8) * 8 * n_chunks;
     DN_CHECK(wgs < ((int64_t)1 << 24), "xg_mu: too many tiles for one launch");
     const dim3 grid((unsigned)wgs), block(256);
-    if (D_out)
+    const bool three = tuning().xg_wgs >= 3.0;  // three workgroups per CU on planes without padding
+    if (three && D_out)
+      hipLaunchKernelGGL((k_xg_mu_tile_b16_w3<true>), grid, block, ABT_LDS64, stream(), X, g_gt, num, eps,
+                         tiles, r, n_chunks, out, D_out);
+    else if (three)
+      hipLaunchKernelGGL((k_xg_mu_tile_b16_w3<false>), grid, block, ABT_LDS64, stream(), X, g_gt, num, eps,
+                         tiles, r, n_chunks, out, D_out);
+    else if (D_out)
       hipLaunchKernelGGL((k_xg_mu_tile_b16<true>), grid, block, ABT_LDS, stream(), X, g_gt, num, eps,
                          tiles, r, n_chunks, out, D_out);
     else

@@ -172,6 +172,7 @@ struct tuning_t {
   double nl_extra_mb = -1.0;       // MB the far tail's slot lists may take beyond their panel copy (-1: 1/128 of the device)
   double nl_lag = 0.0;             // pieces the workgroups of an XCD may be apart
   double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
+  double xg_wgs = 3.0;             // workgroups per CU of the r >= 256 update kernel (2: padded planes, two operand stages)
   double gram_fold = 2.0;          // X^T X on tiles: 2 = diagonal squares of 256 columns in one workgroup where the rank is a
                                    // multiple of 256, else as 1 = diagonal tiles of 128 with their symmetry; 0 = all sixteen blocks
   double nl_wgs = 64.0;            // workgroups of the slot-list kernel per XCD (two per CU)

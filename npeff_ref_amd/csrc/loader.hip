@@ -100,7 +100,7 @@ static const tuning_entry g_tuning_table[] = {
     {"nl_extra_mb", &tuning_t::nl_extra_mb},
     {"nl_spin", &tuning_t::nl_spin},             {"nl_wgs", &tuning_t::nl_wgs},
     {"gram_beside", &tuning_t::gram_beside},
-    {"gram_fold", &tuning_t::gram_fold},
+    {"gram_fold", &tuning_t::gram_fold},         {"xg_wgs", &tuning_t::xg_wgs},
 };
 
 static tuning_t tuning_from_env() {

@@ -128,6 +128,31 @@ def test_xg_mu(rows, r):
     assert np.array_equal(dnum.numpy(), out1)
 
 
+@pytest.mark.parametrize("rows,r", [(128, 256), (4100, 256), (40000, 256), (3000, 512), (700, 1024), (1001, 384)])
+def test_xg_mu_tiles_with_two_and_three_workgroups_per_cu(rows, r, tune):
+    """The update at ranks from 256 on planes without padding (three workgroups per CU, one
+    operand stage, the default) and on padded planes (two, two stages): the same products in the
+    same order, so the same bits, and both within the fp32 bar of the fp64 result."""
+    rng = np.random.default_rng(rows + r)
+    X = (rng.random((rows, r)) * 10.0 ** rng.uniform(-3, 3, size=(1, r))).astype(np.float32)
+    G = rng.random((r, r)).astype(np.float32)
+    num = rng.random((rows, r)).astype(np.float32)
+    eps = np.float32(1e-8)
+    dX, dG, dnum = d.DeviceArray.from_numpy(X), d.DeviceArray.from_numpy(G), d.DeviceArray.from_numpy(num)
+    outs = []
+    for wgs in (3, 2):
+        tune("xg_wgs", wgs)
+        dout, dD = d.DeviceArray((rows, r)), d.DeviceArray((rows, r))
+        d.op_xg_mu(dX, dG, dnum, eps, dout, dD)
+        outs.append((dout.numpy(), dD.numpy()))
+        dout2 = d.DeviceArray((rows, r))
+        d.op_xg_mu(dX, dG, dnum, eps, dout2, None)
+        assert np.array_equal(dout2.numpy(), outs[-1][0])
+    want, wantD = orc.xg_mu_f64(X, G, num, eps)
+    assert _rel(outs[0][1], wantD) < TOL and _rel(outs[0][0], want) < TOL
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+
+
 @pytest.mark.parametrize("split", ["1", "0"])
 @pytest.mark.parametrize("rows", [64, 95, 4100, 70001, 300033])
 def test_xg_mu_gram_fused(rows, split, tune):
