@@ -438,6 +438,10 @@ static int update_H_tiled(dnpeff_nmf* h) {
   DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
   DN_TRY(launch_head_t_product(A, r, h->W));
   DN_TRY(h->prof.end());
+  struct held_g {  // G transposed once for all tiles
+    ~held_g() { xg_mu_release_g(); }
+  } hold;
+  DN_TRY(xg_mu_hold_g(h->G, r));
   for (int64_t q = 0; q < n_tiles; q++) {
     const int64_t t = up ? n_tiles - 1 - q : q;
     const int64_t c0 = t * tile, c1 = c0 + tile < h->m ? c0 + tile : h->m;

@@ -1125,6 +1125,33 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
 // lives until the process ends (one host thread drives the library).
 static float* g_gt = nullptr;
 static int64_t g_gt_floats = 0;
+// The G (and rank) whose transpose g_gt holds for a run of calls, between xg_mu_hold_g and
+// xg_mu_release_g: the column tiles of one H update all multiply by the same G.
+static const float* g_gt_of = nullptr;
+static int g_gt_rank = 0;
+
+static int xg_mu_transpose_g(const float* G, int r) {
+  if (g_gt_floats < (int64_t)r * r) {
+    DN_HIP(hipStreamSynchronize(stream()));
+    dfree(g_gt);
+    g_gt = nullptr;
+    g_gt_floats = 0;
+    g_gt_of = nullptr;
+    DN_TRY(dmalloc(&g_gt, (int64_t)r * r));
+    g_gt_floats = (int64_t)r * r;
+  }
+  return launch_transpose(r, r, G, g_gt);
+}
+
+int xg_mu_hold_g(const float* G, int r) {
+  g_gt_of = nullptr;
+  if (!(use_split_bf16() && r > 128 && r % 128 == 0 && ((uintptr_t)G % 16) == 0)) return 0;  // (no transposed G on that path)
+  DN_TRY(xg_mu_transpose_g(G, r));
+  g_gt_of = G;
+  g_gt_rank = r;
+  return 0;
+}
+void xg_mu_release_g() { g_gt_of = nullptr; }
 
 static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const float* G, const float* num,
                                  float eps, float* out, float* D_out) {
@@ -1136,15 +1163,7 @@ static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const floa
                                hipFuncAttributeMaxDynamicSharedMemorySize, ABT_LDS));
     attr_set = true;
   }
-  if (g_gt_floats < (int64_t)r * r) {
-    DN_HIP(hipStreamSynchronize(stream()));
-    dfree(g_gt);
-    g_gt = nullptr;
-    g_gt_floats = 0;
-    DN_TRY(dmalloc(&g_gt, (int64_t)r * r));
-    g_gt_floats = (int64_t)r * r;
-  }
-  DN_TRY(launch_transpose(r, r, G, g_gt));
+  if (!(g_gt_of == G && g_gt_rank == r)) DN_TRY(xg_mu_transpose_g(G, r));
   const int n_chunks = r / 128;
   const int64_t tiles = rows / 128;
   if (tiles > 0) {

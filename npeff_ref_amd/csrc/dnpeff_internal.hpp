@@ -119,6 +119,10 @@ int launch_gram(int64_t rows, int r, const float* X, float* G, float* workspace)
 // ranks 256, 384, ..., 1024 (head.hip)
 int64_t gram_tiles_workspace_floats(int64_t rows, int r);
 int launch_gram_tiles(int64_t rows, int r, const float* X, float* G, float* workspace);
+// Between the two, launch_xg_mu calls with this G reuse one transposed copy of it (the caller
+// must not change G in between).
+int xg_mu_hold_g(const float* G, int r);
+void xg_mu_release_g();
 int launch_xg_mu(int64_t rows, int r, const float* X, const float* G, const float* num, float eps,
                  float* out, float* D_out);
 // r = 128: the update and the Gram matrix of its output in one pass (dense.hip).
