@@ -14,43 +14,48 @@ using namespace dn;
 // ---------------------------------------------------------------------------
 // Per-kernel timing with HIP events on the library stream
 // ---------------------------------------------------------------------------
-struct EventPair {
-  hipEvent_t start = nullptr, stop = nullptr;
-  int cls = 0;
+// A mark is one event on the stream; the time from a mark to the next one belongs to the class
+// that the mark opens (none for a mark that only closes).  Classes that follow one another
+// without anything between them share the mark between them (next()).
+struct Mark {
+  hipEvent_t ev = nullptr;
+  int cls = -1;
 };
 
 struct Profiler {
   bool enabled = false;
-  std::vector<EventPair> pool;   // every pair ever created
-  size_t used = 0;               // pairs in flight since the last collect
+  std::vector<Mark> pool;        // every event ever created
+  size_t used = 0;               // marks in flight since the last collect
   double ms_sum[DNPEFF_K_COUNT] = {0};
   int64_t launches[DNPEFF_K_COUNT] = {0};
 
-  int begin(int cls) {
-    if (!enabled) return 0;
+  int mark(int cls) {
     if (used == pool.size()) {
-      EventPair p;
-      DN_HIP(hipEventCreate(&p.start));
-      DN_HIP(hipEventCreate(&p.stop));
-      pool.push_back(p);
+      Mark m;
+      DN_HIP(hipEventCreate(&m.ev));
+      pool.push_back(m);
     }
     pool[used].cls = cls;
-    DN_HIP(hipEventRecord(pool[used].start, stream()));
+    DN_HIP(hipEventRecord(pool[used].ev, stream()));
+    used++;
     return 0;
   }
+  int begin(int cls) { return enabled ? mark(cls) : 0; }
+  // closes the open class and opens cls with the same event
+  int next(int cls) { return enabled ? mark(cls) : 0; }
   int end() {
     if (!enabled) return 0;
-    DN_HIP(hipEventRecord(pool[used].stop, stream()));
-    used++;
+    DN_TRY(mark(-1));
     if (used >= 32768) return collect();
     return 0;
   }
   int collect() {
     if (used == 0) return 0;
     DN_HIP(hipStreamSynchronize(stream()));
-    for (size_t i = 0; i < used; i++) {
+    for (size_t i = 0; i + 1 < used; i++) {
+      if (pool[i].cls < 0) continue;
       float ms = 0.0f;
-      DN_HIP(hipEventElapsedTime(&ms, pool[i].start, pool[i].stop));
+      DN_HIP(hipEventElapsedTime(&ms, pool[i].ev, pool[i + 1].ev));
       ms_sum[pool[i].cls] += (double)ms;
       launches[pool[i].cls] += 1;
     }
@@ -64,10 +69,8 @@ struct Profiler {
     }
   }
   ~Profiler() {
-    for (auto& p : pool) {
-      if (p.start) (void)hipEventDestroy(p.start);
-      if (p.stop) (void)hipEventDestroy(p.stop);
-    }
+    for (auto& m : pool)
+      if (m.ev) (void)hipEventDestroy(m.ev);
   }
 };
 
@@ -445,13 +448,13 @@ static int update_H_tiled(dnpeff_nmf* h) {
   for (int64_t q = 0; q < n_tiles; q++) {
     const int64_t t = up ? n_tiles - 1 - q : q;
     const int64_t c0 = t * tile, c1 = c0 + tile < h->m ? c0 + tile : h->m;
-    DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+    // (one event per change of class: a tile's product starts where the tile before ended)
+    DN_TRY(q == 0 ? h->prof.begin(DNPEFF_K_SPMM_T) : h->prof.next(DNPEFF_K_SPMM_T));
     DN_TRY(launch_spmm_t_tile(A, r, h->W, c0, c1, h->S));
-    DN_TRY(h->prof.end());
-    DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_H));
+    DN_TRY(h->prof.next(DNPEFF_K_XG_MU_H));
     DN_TRY(launch_xg_mu(c1 - c0, r, h->H + c0 * r, h->G, h->S, h->eps, Hnew + c0 * r, nullptr));
-    DN_TRY(h->prof.end());
   }
+  DN_TRY(h->prof.end());
   h->H = Hnew;
   h->gh_valid = false;
   return 0;
