@@ -77,6 +77,8 @@ int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int
 /* Switches for experiments and for tests that must reach a particular code path; no counterpart
  * in the reference.  Names: dense_fill, panels, sweep_bytes, sweep_min, sweep_waves, sweep_lag,
  * sweep_spin, spmm_t_slices, split_bf16, fused_gram, h_tile_mb, tiled_h, topk_fast_cap, verbose,
+ * h_overlap (1: tiled H update with A^T W of the next tile on the library stream beside the
+ * update of this tile on a second stream, through two tile buffers; off by default),
  * xg_wgs (3: the update kernel of ranks from 256 with three workgroups per CU on LDS planes
  * without padding; 2: two, on padded planes with two operand stages),
  * gram_beside (H^T H of the W update on a second stream beside A H^T), gram_fold (2: X^T X with

@@ -88,6 +88,7 @@ struct dnpeff_nmf {
   float* Nw = nullptr;       // [n, r] A H^T
   float* H = nullptr;        // [m, r] (points into Hbuf)
   float* S = nullptr;        // [m, r] A^T W, then the updated H; tiled: [tile_cols, r], A^T W of a tile
+  float* S2 = nullptr;       // tiled, h_overlap: a second tile buffer
   float* Hbuf = nullptr;     // allocation that holds H; tiled: [m + tile_cols, r]
   // Tiled H update (when a second [m, r] array does not fit): A^T W is formed for tile_cols
   // columns at a time and the updated tile is written one tile below (or above) the place of the
@@ -110,7 +111,7 @@ struct dnpeff_nmf {
 DN_API int dnpeff_nmf_destroy(dnpeff_nmf* nmf) {
   if (!nmf) return 0;
   (void)hipStreamSynchronize(stream());
-  dfree(nmf->W); dfree(nmf->W2); dfree(nmf->Nw); dfree(nmf->Hbuf); dfree(nmf->S);
+  dfree(nmf->W); dfree(nmf->W2); dfree(nmf->Nw); dfree(nmf->Hbuf); dfree(nmf->S); dfree(nmf->S2);
   dfree(nmf->G); dfree(nmf->G2); dfree(nmf->gram_ws); dfree(nmf->dot_ws);
   dfree(nmf->GH); dfree(nmf->gpart);
   delete nmf;
@@ -315,6 +316,7 @@ static int nmf_create_impl(dnpeff_csr* A, int rank, float eps, int64_t seed, uns
   h->H = h->Hbuf;
   if (!s && fused_update(h))
     s = dmalloc(&h->GH, (int64_t)rank * rank) || dmalloc(&h->gpart, xg_mu_gram_workspace_floats(h->m));
+  if (!s && h->tiled && tuning().h_overlap != 0.0) s = dmalloc(&h->S2, s_floats);
   if (!s && h->tiled) s = csr_tile_lists(A);
   if (s) { dnpeff_nmf_destroy(h); return s; }
   mark("factors and workspaces");
@@ -432,7 +434,62 @@ DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
 // the tiles are walked from the last to the first (a new tile then lands on old tiles that were
 // read already); H one tile up: the new H goes to the start, first tile first.  The tiles are
 // independent of one another, so the order does not change any sum.
+// The same with A^T W of tile q + 1 (library stream) running beside the update of tile q (second
+// stream of the same priority), through two tile buffers.  The updates follow one another on
+// their stream, so the rule about where a new tile may land holds as it does above; a product
+// waits for the update that last read its buffer.  Same kernels on the same operands: same bits.
+static int update_H_tiled_overlapped(dnpeff_nmf* h) {
+  dnpeff_csr* A = h->A;
+  const int r = h->r;
+  const int64_t tile = h->tile_cols, n_tiles = ceil_div(h->m, tile);
+  const bool up = h->H == h->Hbuf;
+  float* Hnew = up ? h->Hbuf + tile * r : h->Hbuf;
+  static hipEvent_t ev_t[2] = {nullptr, nullptr}, ev_x[2] = {nullptr, nullptr}, fork = nullptr;
+  if (!fork) {
+    DN_HIP(hipEventCreateWithFlags(&fork, hipEventDisableTiming));
+    for (int b = 0; b < 2; b++) {
+      DN_HIP(hipEventCreateWithFlags(&ev_t[b], hipEventDisableTiming));
+      DN_HIP(hipEventCreateWithFlags(&ev_x[b], hipEventDisableTiming));
+    }
+  }
+  hipStream_t s0 = stream(), s1 = side_stream_handle();
+  DN_CHECK(s1 != nullptr, "second stream");
+  struct guard {  // whatever happens, the library stream is where later launches go
+    ~guard() { side_stream_route(false); xg_mu_release_g(); }
+  } g;
+  DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+  DN_TRY(launch_head_t_product(A, r, h->W));
+  DN_TRY(h->prof.end());
+  DN_TRY(xg_mu_hold_g(h->G, r));
+  DN_HIP(hipEventRecord(fork, s0));
+  DN_HIP(hipStreamWaitEvent(s1, fork, 0));
+  for (int64_t q = 0; q < n_tiles; q++) {
+    const int64_t t = up ? n_tiles - 1 - q : q;
+    const int64_t c0 = t * tile, c1 = c0 + tile < h->m ? c0 + tile : h->m;
+    const int b = (int)(q & 1);
+    float* Sb = b ? h->S2 : h->S;
+    if (q >= 2) DN_HIP(hipStreamWaitEvent(s0, ev_x[b], 0));
+    DN_TRY(h->prof.begin(DNPEFF_K_SPMM_T));
+    DN_TRY(launch_spmm_t_tile(A, r, h->W, c0, c1, Sb));
+    DN_TRY(h->prof.end());
+    DN_HIP(hipEventRecord(ev_t[b], s0));
+    DN_HIP(hipStreamWaitEvent(s1, ev_t[b], 0));
+    side_stream_route(true);
+    DN_TRY(h->prof.begin(DNPEFF_K_XG_MU_H));
+    DN_TRY(launch_xg_mu(c1 - c0, r, h->H + c0 * r, h->G, Sb, h->eps, Hnew + c0 * r, nullptr));
+    DN_TRY(h->prof.end());
+    side_stream_route(false);
+    DN_HIP(hipEventRecord(ev_x[b], s1));
+  }
+  DN_HIP(hipStreamWaitEvent(s0, ev_x[0], 0));
+  if (n_tiles > 1) DN_HIP(hipStreamWaitEvent(s0, ev_x[1], 0));
+  h->H = Hnew;
+  h->gh_valid = false;
+  return 0;
+}
+
 static int update_H_tiled(dnpeff_nmf* h) {
+  if (h->S2) return update_H_tiled_overlapped(h);
   dnpeff_csr* A = h->A;
   const int r = h->r;
   const int64_t tile = h->tile_cols, n_tiles = ceil_div(h->m, tile);

@@ -25,6 +25,8 @@ int n_cus();
 int side_stream_begin();
 int side_stream_end();
 int side_stream_join();
+hipStream_t side_stream_handle();
+void side_stream_route(bool on);
 
 }  // namespace dn
 
@@ -176,6 +178,7 @@ struct tuning_t {
   double nl_extra_mb = -1.0;       // MB the far tail's slot lists may take beyond their panel copy (-1: 1/128 of the device)
   double nl_lag = 0.0;             // pieces the workgroups of an XCD may be apart
   double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
+  double h_overlap = 0.0;          // tiled H update: A^T W of the next tile beside the update of this one (two streams, two tile buffers)
   double xg_wgs = 3.0;             // workgroups per CU of the r >= 256 update kernel (2: padded planes, two operand stages)
   double gram_fold = 2.0;          // X^T X on tiles: 2 = diagonal squares of 256 columns in one workgroup where the rank is a
                                    // multiple of 256, else as 1 = diagonal tiles of 128 with their symmetry; 0 = all sixteen blocks

@@ -74,6 +74,14 @@ int side_stream_join() {
   return 0;
 }
 
+// The two streams by themselves, and where stream() points, for callers that order work between
+// them with events of their own.
+hipStream_t side_stream_handle() {
+  if (!g_side_stream && hipStreamCreate(&g_side_stream) != hipSuccess) return nullptr;
+  return g_side_stream;
+}
+void side_stream_route(bool on) { g_on_side_stream = on && g_side_stream != nullptr; }
+
 int n_cus() {
   if (!g_n_cus) {
     hipDeviceProp_t p;
@@ -101,6 +109,7 @@ static const tuning_entry g_tuning_table[] = {
     {"nl_spin", &tuning_t::nl_spin},             {"nl_wgs", &tuning_t::nl_wgs},
     {"gram_beside", &tuning_t::gram_beside},
     {"gram_fold", &tuning_t::gram_fold},         {"xg_wgs", &tuning_t::xg_wgs},
+    {"h_overlap", &tuning_t::h_overlap},
 };
 
 static tuning_t tuning_from_env() {

@@ -368,6 +368,38 @@ def _steps(A, r, seed, steps, consume=False):
     return nmf
 
 
+@pytest.mark.parametrize("r,n,k,tile_mb", [(256, 1100, 3000, 0.9), (64, 300, 2000, 0.05), (512, 300, 2500, 1.5)])
+def test_tiled_H_update_with_the_next_product_beside_it(r, n, k, tile_mb, tune):
+    """`h_overlap`: A^T W of tile q + 1 on the library stream beside the update of tile q on a
+    second stream, through two tile buffers.  Same kernels on the same operands in an order that
+    the events between the streams fix: the same bits as the tiled update on one stream, after
+    odd and even numbers of steps, and the calls that follow (loss, factors to the host) see
+    the finished update."""
+    tune("fused_gram", 0)
+    tune("tiled_h", 1)
+    tune("h_tile_mb", tile_mb)
+    seed = 300 + r
+    A, norms = d.Csr.synth(n, 60000, k_fixed=k, zipf_s=1.2, seed=seed)
+    A.normalize_rows(norms)
+    A.compact_columns(1)
+    ref = _steps(A, r, seed, 3)
+    tiled, tile_cols = ref.info()
+    assert tiled and 3 * tile_cols < A.n_cols
+    W3, H3, loss3 = ref.loadWToHostSync(), ref.loadHToHostSync(), ref.computeUncachedLoss()
+    ref.step(2)
+    W5, H5, loss5 = ref.loadWToHostSync(), ref.loadHToHostSync(), ref.computeUncachedLoss()
+    ref.close()
+    tune("h_overlap", 1)
+    ovl = _steps(A, r, seed, 3)
+    assert ovl.info() == (tiled, tile_cols)
+    assert np.array_equal(ovl.loadWToHostSync(), W3) and np.array_equal(ovl.loadHToHostSync(), H3)
+    assert ovl.computeUncachedLoss() == loss3
+    ovl.step(2)
+    assert np.array_equal(ovl.loadWToHostSync(), W5) and np.array_equal(ovl.loadHToHostSync(), H5)
+    assert ovl.computeUncachedLoss() == loss5
+    ovl.close()
+
+
 @pytest.mark.parametrize("r,n,k,tile_mb", [(256, 1100, 3000, 0.9), (128, 1100, 3000, 0.4), (64, 300, 2000, 0.05),
                                            (48, 130, 800, 0.03)])
 def test_tiled_H_update_gives_the_same_bits(r, n, k, tile_mb, tune):
