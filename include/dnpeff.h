@@ -81,7 +81,8 @@ int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int
  * update of this tile on a second stream, through two tile buffers; off by default),
  * xg_wgs (3: the update kernel of ranks from 256 with three workgroups per CU on LDS planes
  * without padding; 2: two, on padded planes with two operand stages),
- * gram_beside (H^T H of the W update on a second stream beside A H^T), gram_fold (2: X^T X with
+ * gram_beside (1: H^T H of the W update on a second stream with the dense head of A H^T behind
+ * it; 0: after A H^T on the library stream), gram_fold (2: X^T X with
  * its diagonal squares of 256 columns each in one workgroup where the rank is a multiple of 256;
  * 1: diagonal tiles of 128 columns with their symmetry used; 0: without), n_lists (A H^T from slot lists on component slices of 32: -1 =
  * the far tail of the sparse part where that was measured to pay, 2 = wherever possible, 1 = the

@@ -20,6 +20,7 @@ using namespace dn;
 struct Mark {
   hipEvent_t ev = nullptr;
   int cls = -1;
+  bool counts = true;  // the segment is a launch of its class (not the continuation of one)
 };
 
 struct Profiler {
@@ -29,18 +30,21 @@ struct Profiler {
   double ms_sum[DNPEFF_K_COUNT] = {0};
   int64_t launches[DNPEFF_K_COUNT] = {0};
 
-  int mark(int cls) {
+  int mark(int cls, bool counts = true) {
     if (used == pool.size()) {
       Mark m;
       DN_HIP(hipEventCreate(&m.ev));
       pool.push_back(m);
     }
     pool[used].cls = cls;
+    pool[used].counts = counts;
     DN_HIP(hipEventRecord(pool[used].ev, stream()));
     used++;
     return 0;
   }
   int begin(int cls) { return enabled ? mark(cls) : 0; }
+  // goes on with a class that was interrupted (its time, not another launch)
+  int resume(int cls) { return enabled ? mark(cls, false) : 0; }
   // closes the open class and opens cls with the same event
   int next(int cls) { return enabled ? mark(cls) : 0; }
   int end() {
@@ -56,8 +60,9 @@ struct Profiler {
       if (pool[i].cls < 0) continue;
       float ms = 0.0f;
       DN_HIP(hipEventElapsedTime(&ms, pool[i].ev, pool[i + 1].ev));
+      if (ms < 0.0f) ms = 0.0f;  // (marks on two streams: the later mark's work ended first)
       ms_sum[pool[i].cls] += (double)ms;
-      launches[pool[i].cls] += 1;
+      if (pool[i].counts) launches[pool[i].cls] += 1;
     }
     used = 0;
     return 0;
@@ -391,16 +396,33 @@ static int products_for(dnpeff_nmf* h) {
 DN_API int dnpeff_nmf_update_W(dnpeff_nmf* h) {
   DN_CHECK(h != nullptr, "handle is NULL");
   dnpeff_csr* A = h->A;
-  // H^T H and A H^T both only read H: with the gram_beside switch the Gram kernel (bound by
-  // instruction issue) runs on a second stream beside the head product and the plain panels of
-  // A H^T (bound by the fabric)
   bool gram_done = false;
   if (!h->nw_valid && !h->gh_valid && tuning().gram_beside != 0.0) {
+    // H^T H on the second stream, the dense head of A H^T on the library stream behind it: the
+    // head's workgroups take the CUs as those of H^T H leave them, and the rest of A H^T (kernels
+    // that need the whole chip) starts when both are done.  Timing: H^T H from its start to its
+    // end; A H^T from the end of H^T H to the end of the head (what the head adds), then the rest.
+    DN_TRY(products_for(h));
+    struct guard {
+      ~guard() { side_stream_route(false); }
+    } g;
     DN_TRY(side_stream_begin());
-    int st = launch_gram(h->m, h->r, h->H, h->G, h->gram_ws);
+    int st = h->prof.begin(DNPEFF_K_GRAM_H);
+    if (!st) st = launch_gram(h->m, h->r, h->H, h->G, h->gram_ws);
+    if (!st) st = h->prof.next(DNPEFF_K_SPMM_N);
     DN_TRY(side_stream_end());
     DN_TRY(st);
     gram_done = true;
+    DN_TRY(launch_spmm_n(A, h->r, h->H, 1));
+    DN_TRY(h->prof.end());
+    DN_TRY(side_stream_join());
+    DN_TRY(h->prof.resume(DNPEFF_K_SPMM_N));
+    DN_TRY(launch_spmm_n(A, h->r, h->H, 2));
+    DN_TRY(h->prof.end());
+    DN_TRY(h->prof.begin(DNPEFF_K_SPMM_N_REDUCE));
+    DN_TRY(launch_spmm_n_reduce(A, h->r, h->Nw));
+    DN_TRY(h->prof.end());
+    h->nw_valid = true;
   }
   if (!h->nw_valid) {  // a loss evaluation since the last H update has left A H^T in Nw
     DN_TRY(products_for(h));

@@ -145,7 +145,7 @@ constexpr int64_t SPMM_N_CHUNK = 2048;  // entries of one row handled by one wor
 constexpr int64_t SPMM_T_LONG = 256;    // columns longer than this get a whole workgroup
 // A H^T in two steps (partial sums, then their reduction); both cover the sparse part and the
 // dense head of A.  Need csr_ensure_products(A, r).
-int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr);
+int launch_spmm_n(const dnpeff_csr* A, int r, const float* H_mr, int part = 0);
 int launch_spmm_n_reduce(const dnpeff_csr* A, int r, float* N_nr);
 int launch_spmm_t(const dnpeff_csr* A, int r, const float* W_nr, float* T_mr);
 int launch_spsp(const dnpeff_csr* A, dnpeff_csr* B, float* partials);
@@ -177,7 +177,7 @@ struct tuning_t {
   double nl_piece_cols = 32768.0;  // columns per piece of the slot lists
   double nl_extra_mb = -1.0;       // MB the far tail's slot lists may take beyond their panel copy (-1: 1/128 of the device)
   double nl_lag = 0.0;             // pieces the workgroups of an XCD may be apart
-  double gram_beside = 0.0;        // H^T H of the W update on a second stream beside the plain panels of A H^T (1 = on)
+  double gram_beside = 1.0;        // H^T H of the W update on a second stream beside the dense head and the plain panels of A H^T (0 = after A H^T)
   double h_overlap = 0.0;          // tiled H update: A^T W of the next tile beside the update of this one (two streams, two tile buffers)
   double xg_wgs = 3.0;             // workgroups per CU of the r >= 256 update kernel (2: padded planes, two operand stages)
   double gram_fold = 2.0;          // X^T X on tiles: 2 = diagonal squares of 256 columns in one workgroup where the rank is a

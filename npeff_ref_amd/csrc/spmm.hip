@@ -1177,11 +1177,18 @@ static int launch_spmm_n_sweep(const dnpeff_csr* A, int r, const float* H_mr, bo
   return 0;
 }
 
-int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
+// part: 0 = the whole product; 1 = what may run beside another kernel: the dense head, and the
+// plain panels where they are the far tail (no slot lists: a long kernel that waits for the
+// fabric); 2 = the rest (swept pieces and slot lists, whose workgroups walk in lock step and
+// must all be resident; everything, where the product is not planned in panels).  1 then 2
+// launch what 0 launches, in the same order.
+int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr, int part) {
   DN_CHECK(r >= 1 && r <= MAX_RANK, "rank %d outside [1, %d]", r, MAX_RANK);
-  DN_TRY(launch_head_n(A_full, r, H_mr));
+  if (part != 2) DN_TRY(launch_head_n(A_full, r, H_mr));
   const dnpeff_csr* A = sparse_part(A_full);
   float* partials = A->partials;
+  const bool planned = !(A->nl.pairs && use_nlists(A, r)) && A->n_panels > 0;
+  if (part == 1 && !planned) return 0;
   if (A->nl.pairs && use_nlists(A, r)) {
     DN_CHECK(partials && A->partials_floats >= A->n_rows * (int64_t)r, "partial sums too small");
     return launch_spmm_n_lists(A, r, H_mr, partials, r);
@@ -1190,7 +1197,8 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
     DN_CHECK(A->seg && A->pcol && A->panel_ids && partials, "matrix has no panel work list");
     const bool aligned = ((uintptr_t)H_mr % 16) == 0;
     const int slots = (int)panel_slots(A);
-    if (A->n_plain > 0) {
+    const bool plain_early = A->tail_floor == 0;  // (in part 1)
+    if (A->n_plain > 0 && (part == 0 || (part == 1) == plain_early)) {
       const int64_t row_groups = ceil_div(A->n_rows, 4);
       dim3 grid((unsigned)(row_groups * A->n_plain)), block(256);
       dispatch_gather(r, aligned, [&](auto tag) {
@@ -1202,6 +1210,7 @@ int launch_spmm_n(const dnpeff_csr* A_full, int r, const float* H_mr) {
       });
       DN_LAUNCH_CHECK();
     }
+    if (part == 1) return 0;
     // (the sweep kernel wants the CUs to itself: all its workgroups must be resident)
     if (A->n_swept > 0) {
       DN_TRY(side_stream_join());
