@@ -80,7 +80,8 @@ int dnpeff_plan_estimate(int64_t n_rows, int64_t n_cols, int64_t nnz_sparse, int
  * h_overlap (1: tiled H update with A^T W of the next tile on the library stream beside the
  * update of this tile on a second stream, through two tile buffers; off by default),
  * xg_wgs (3: the update kernel of ranks from 256 with three workgroups per CU on LDS planes
- * without padding; 2: two, on padded planes with two operand stages),
+ * without padding where the launch fills the CUs eight times over; 4: always; 2: two, on padded
+ * planes with two operand stages),
  * gram_beside (1: H^T H of the W update on a second stream with the dense head of A H^T behind
  * it; 0: after A H^T on the library stream), gram_fold (2: X^T X with
  * its diagonal squares of 256 columns each in one workgroup where the rank is a multiple of 256;

@@ -1170,7 +1170,10 @@ static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const floa
     const int64_t wgs = ceil_div(tiles, 8) * 8 * n_chunks;
     DN_CHECK(wgs < ((int64_t)1 << 24), "xg_mu: too many tiles for one launch");
     const dim3 grid((unsigned)wgs), block(256);
-    const bool three = tuning().xg_wgs >= 3.0;  // three workgroups per CU on planes without padding
+    // three workgroups per CU on planes without padding, where the launch fills them several
+    // times over (a workgroup of three takes longer than one of two: few row tiles, as in the
+    // fixed-H learner's W update, are done sooner two per CU)
+    const bool three = tuning().xg_wgs >= 4.0 || (tuning().xg_wgs >= 3.0 && wgs >= 8 * 3 * (int64_t)n_cus());
     if (three && D_out)
       hipLaunchKernelGGL((k_xg_mu_tile_b16_w3<true>), grid, block, ABT_LDS64, stream(), X, g_gt, num, eps,
                          tiles, r, n_chunks, out, D_out);

@@ -179,7 +179,7 @@ struct tuning_t {
   double nl_lag = 0.0;             // pieces the workgroups of an XCD may be apart
   double gram_beside = 1.0;        // H^T H of the W update on a second stream beside the dense head and the plain panels of A H^T (0 = after A H^T)
   double h_overlap = 0.0;          // tiled H update: A^T W of the next tile beside the update of this one (two streams, two tile buffers)
-  double xg_wgs = 3.0;             // workgroups per CU of the r >= 256 update kernel (2: padded planes, two operand stages)
+  double xg_wgs = 3.0;             // workgroups per CU of the r >= 256 update kernel: 3 where the launch fills the CUs eight times, 4 = three always, 2 = two (padded planes, two operand stages)
   double gram_fold = 2.0;          // X^T X on tiles: 2 = diagonal squares of 256 columns in one workgroup where the rank is a
                                    // multiple of 256, else as 1 = diagonal tiles of 128 with their symmetry; 0 = all sixteen blocks
   double nl_wgs = 64.0;            // workgroups of the slot-list kernel per XCD (two per CU)

@@ -128,7 +128,8 @@ def test_xg_mu(rows, r):
     assert np.array_equal(dnum.numpy(), out1)
 
 
-@pytest.mark.parametrize("rows,r", [(128, 256), (4100, 256), (40000, 256), (3000, 512), (700, 1024), (1001, 384)])
+@pytest.mark.parametrize("rows,r", [(128, 256), (4100, 256), (40000, 256), (3000, 512), (700, 1024), (1001, 384),
+                                    (400000, 256)])
 def test_xg_mu_tiles_with_two_and_three_workgroups_per_cu(rows, r, tune):
     """The update at ranks from 256 on planes without padding (three workgroups per CU, one
     operand stage, the default) and on padded planes (two, two stages): the same products in the
@@ -140,7 +141,7 @@ def test_xg_mu_tiles_with_two_and_three_workgroups_per_cu(rows, r, tune):
     eps = np.float32(1e-8)
     dX, dG, dnum = d.DeviceArray.from_numpy(X), d.DeviceArray.from_numpy(G), d.DeviceArray.from_numpy(num)
     outs = []
-    for wgs in (3, 2):
+    for wgs in (4, 2):  # (4: three per CU whatever the size; 3, the default, only for launches that fill the CUs eight times)
         tune("xg_wgs", wgs)
         dout, dD = d.DeviceArray((rows, r)), d.DeviceArray((rows, r))
         d.op_xg_mu(dX, dG, dnum, eps, dout, dD)
@@ -151,6 +152,10 @@ def test_xg_mu_tiles_with_two_and_three_workgroups_per_cu(rows, r, tune):
     want, wantD = orc.xg_mu_f64(X, G, num, eps)
     assert _rel(outs[0][1], wantD) < TOL and _rel(outs[0][0], want) < TOL
     assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    tune("xg_wgs", 3)
+    dout = d.DeviceArray((rows, r))
+    d.op_xg_mu(dX, dG, dnum, eps, dout, None)
+    assert np.array_equal(dout.numpy(), outs[0][0])
 
 
 @pytest.mark.parametrize("split", ["1", "0"])
