@@ -560,9 +560,11 @@ def run_fit(d, args, cfg):
     hist = []
     elapsed = 0.0
     t0 = time.perf_counter()
+    log_every = 25  # log_every_n_steps (only_W_learner_params.h:35); the loss is not timed
     for i in range(steps):
-        L.step(1)
-        if (i + 1) % 25 == 0:  # log_every_n_steps (only_W_learner_params.h:35); the loss is not timed
+        if i % log_every == 0:  # the steps up to the next logged one in one call of the library
+            L.step(min(log_every, steps - i))
+        if (i + 1) % log_every == 0:
             d.sync()
             elapsed += time.perf_counter() - t0
             hist.append((i + 1,) + L.losses())

@@ -776,6 +776,10 @@ DN_API int dnpeff_fit_set_W(dnpeff_fit* f, const float* W_nr) {
 DN_API int dnpeff_fit_step(dnpeff_fit* f, int n_steps) {
   clear_error();
   DN_CHECK(f != nullptr, "handle is NULL");
+  struct held_g {  // H H^T is the same in every step: one transposed copy for all of them
+    ~held_g() { xg_mu_release_g(); }
+  } hold;
+  DN_TRY(xg_mu_hold_g(f->HH, f->r));
   for (int s = 0; s < n_steps; s++) {
     DN_TRY(launch_xg_mu(f->n, f->r, f->W, f->HH, f->AH, f->eps, f->W2, f->WHH));
     std::swap(f->W, f->W2);

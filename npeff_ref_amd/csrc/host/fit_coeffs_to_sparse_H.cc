@@ -119,8 +119,14 @@ int main(int argc, char** argv) {
   ck(dnpeff_fit_init_W(fit));
   ck(dnpeff_sync());
   auto t_start = std::chrono::high_resolution_clock::now();
-  for (long i = 0; i < flags.max_iters; i++) {
-    ck(dnpeff_fit_step(fit, 1));
+  // the steps up to the next logged one in one call (the library then prepares H H^T once for all
+  // of them); the sequence of updates is the loop's, one step at a time
+  for (long i = 0; i < flags.max_iters;) {
+    long run = flags.max_iters - i;
+    if (flags.log_every > 0 && run > flags.log_every - i % flags.log_every) run = flags.log_every - i % flags.log_every;
+    if (run > 1000000) run = 1000000;
+    ck(dnpeff_fit_step(fit, (int)run));
+    i += run - 1;
     if (flags.log_every > 0 && ((i + 1) % flags.log_every) == 0) {
       ck(dnpeff_sync());
       auto t_end = std::chrono::high_resolution_clock::now();
@@ -131,6 +137,7 @@ int main(int argc, char** argv) {
                 << elapsed_ms / (double)flags.log_every << " ms/step]\n";
       t_start = std::chrono::high_resolution_clock::now();
     }
+    i++;
   }
   ck(dnpeff_sync());
   std::cout << "Finished running second stage.\n";
