@@ -1166,6 +1166,18 @@ static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const floa
   if (!(g_gt_of == G && g_gt_rank == r)) DN_TRY(xg_mu_transpose_g(G, r));
   const int n_chunks = r / 128;
   const int64_t tiles = rows / 128;
+  // The last rows (fewer than 128, through the fp32 kernel: two workgroups that take a third of
+  // the time of a few hundred row tiles) run on the second stream beside the whole tiles.
+  const int64_t head = tiles * 128;
+  bool beside = false;
+  if (head < rows && tiles > 0 && tiles <= 4096 && !side_stream_routed() && !side_stream_pending()) {
+    DN_TRY(side_stream_begin());
+    const int64_t off = head * r;
+    int st = launch_xg_mu_tile(rows - head, r, X + off, G, num + off, eps, out + off, D_out ? D_out + off : nullptr);
+    DN_TRY(side_stream_end());
+    DN_TRY(st);
+    beside = true;
+  }
   if (tiles > 0) {
     const int64_t wgs = ceil_div(tiles, 8) * 8 * n_chunks;
     DN_CHECK(wgs < ((int64_t)1 << 24), "xg_mu: too many tiles for one launch");
@@ -1188,7 +1200,7 @@ static int launch_xg_mu_tile_b16(int64_t rows, int r, const float* X, const floa
                          tiles, r, n_chunks, out, D_out);
     DN_LAUNCH_CHECK();
   }
-  const int64_t head = tiles * 128;
+  if (beside) return side_stream_join();
   if (head < rows) {
     const int64_t off = head * r;
     DN_TRY(launch_xg_mu_tile(rows - head, r, X + off, G, num + off, eps, out + off,

@@ -27,6 +27,8 @@ int side_stream_end();
 int side_stream_join();
 hipStream_t side_stream_handle();
 void side_stream_route(bool on);
+bool side_stream_routed();
+bool side_stream_pending();
 
 }  // namespace dn
 

@@ -81,6 +81,8 @@ hipStream_t side_stream_handle() {
   return g_side_stream;
 }
 void side_stream_route(bool on) { g_on_side_stream = on && g_side_stream != nullptr; }
+bool side_stream_routed() { return g_on_side_stream; }
+bool side_stream_pending() { return g_side_done != nullptr; }
 
 int n_cus() {
   if (!g_n_cus) {
