@@ -369,7 +369,9 @@ int dnpeff_fit_init_W(dnpeff_fit* fit);
 int dnpeff_fit_set_W(dnpeff_fit* fit, const float* W_nr);
 
 /* n_steps of WHH = W (H H^T); W <- W * (A H^T) / (WHH + eps)
- * (DoMuStep, nmf_sparse_H.h:342-345). */
+ * (DoMuStep, nmf_sparse_H.h:342-345).  Several steps in one call give the same W as as many
+ * calls of one step, and cost less: what the steps share (H H^T in the layout the kernel reads)
+ * is prepared once per call. */
 int dnpeff_fit_step(dnpeff_fit* fit, int n_steps);
 
 /* reference_loss: sqrt(||A||^2 + <WHH, W> - 2 <A H^T, W>) with WHH as left by
