@@ -225,6 +225,40 @@ def test_fit_path_first_stage_and_loop():
     H.close()
 
 
+@pytest.mark.parametrize("n", [2000 + 80, 1024])
+def test_fit_steps_in_one_call_and_one_by_one_rank_256(n):
+    """The W loop of the fixed-H learner at rank 256 (matrix-core update kernel; with n = 2080 the
+    last 32 rows go through another kernel, on the second stream): seven steps in one call, seven
+    calls of one step and a 3 + 4 split give the same W bit for bit, and the oracle's within the
+    bar."""
+    rng = np.random.default_rng(n)
+    m, r, eps = 30000, 256, 1e-7
+    ar, ac, av, norms = d.synth_pef_host(n, m, k_fixed=600, seed=8)
+    av = orc.normalize_rows(ar, av, norms)
+    b = random_csr(rng, r, m, 700, sort_cols=True)
+    A, H = d.Csr.from_host(ar, ac, av, m), d.Csr.from_host(*b, m)
+    lrn = d.Learner(A, H, d.LearnerParams(max_iters=7, eps=eps, log_every_n_steps=0))
+    AH, HH, sq = lrn.products()
+    lrn.initialize()
+    W0 = lrn.GetOnHost_W()
+    lrn.step(7)
+    W7 = lrn.GetOnHost_W()
+    lrn.set_W(W0)
+    for _ in range(7):
+        lrn.step(1)
+    assert np.array_equal(lrn.GetOnHost_W(), W7)
+    lrn.set_W(W0)
+    lrn.step(3)
+    lrn.losses()
+    lrn.step(4)
+    assert np.array_equal(lrn.GetOnHost_W(), W7)
+    W64, _, _ = orc.fit_f64(AH.astype(np.float64), HH.astype(np.float64), sq, W0, np.float32(eps), 7, 0)
+    assert _nrm(W7, W64) < REL
+    lrn.close()
+    A.close()
+    H.close()
+
+
 def test_dense_head_run_matches_oracle_and_unsplit_run(tune):
     """n >= 1024 rows and r >= 64: dnpeff_nmf_create moves the columns most rows hold into the
     dense block by itself; the run stays within the bar of the fp64 oracle and close to the run
