@@ -99,10 +99,11 @@ def test_run_is_reproducible_bit_for_bit():
     assert outs[0][2] == outs[1][2]
 
 
-@pytest.mark.parametrize("rank", [64, 128])
+@pytest.mark.parametrize("rank", [64, 128, 256])
 def test_loss_evaluations_do_not_change_the_run(rank):
     """The loss leaves A H^T behind for the next W update (and takes H^T H from the fused H update
-    at rank 128): a run that evaluates the loss after every step and between the two updates ends
+    at rank 128; at rank 256 a W update that finds A H^T there does not start H^T H on the second
+    stream): a run that evaluates the loss after every step and between the two updates ends
     on the same bits as one that never does, and the loss values agree with a fresh evaluation."""
     outs = []
     for with_loss in (False, True):
