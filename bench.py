@@ -469,6 +469,10 @@ def run_nmf(d, args, cfg):
                    "zipf_s": cfg["s"], "rank": r, "eps": args.eps, "seed": args.seed,
                    "dense_head_columns": n_dense, "nnz_sparse_part": z_sparse, "tiled_H_update": tiled,
                    "H_tile_columns": tile_cols, "sparse_part_of_A_Ht": sparse_plan,
+                   "H_gram_in_W_update": ("second stream, ahead of the dense head of A H^T; the class times count "
+                                          "the time both run only once (under gram_H)"
+                                          if d.tuning_get("gram_beside") != 0.0 and not fused_gram
+                                          else "library stream"),
                    "device_memory_used_gb": (total - free1) / 1e9,
                    "device_memory_total_gb": total / 1e9},
         "roofline": roofline,
